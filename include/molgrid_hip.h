@@ -1,0 +1,157 @@
+/*
+ * molgrid_hip.h -- C ABI of the MI355X (gfx950) gridding kernels.
+ *
+ * This is the drop-in boundary of the gridding hot path: the host-side
+ * GridMaker / Transform / GridInterpolater classes (C++ and Python) validate
+ * their arguments exactly as the reference does and then call one of these
+ * entry points where the reference launched its CUDA kernels.  Signatures use
+ * plain pointers and sizes only.
+ *
+ * Conventions
+ *   - Every array pointer is a DEVICE pointer on the current HIP device unless
+ *     its name ends in `_host`.  Arrays are dense, row-major, float32.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Work
+ *     is enqueued asynchronously; no entry point synchronises or allocates.
+ *   - Batches: example b owns atoms [atom_offsets[b], atom_offsets[b+1]) of the
+ *     packed atom arrays.  When `atom_offsets` is NULL every example owns
+ *     `atoms_per_example` consecutive atoms (the reference's padded BxN layout,
+ *     include/libmolgrid/grid_maker.h:265-301; nbatch = 1 is the un-batched
+ *     call).  Per-example float3/float4 parameters (`centers`, `quats`, ...)
+ *     are device arrays with one row per example; when such a pointer is NULL
+ *     the `_host` value beside it is used for every example.
+ *   - Return value: MG_OK, a negative MG_ERR_* code for a rejected argument
+ *     (nothing was launched), or a positive hipError_t from the launch.
+ *   - Atoms with a negative type index are ignored.  A type index >= ntypes is
+ *     ignored as well (the reference's CPU overload throws std::out_of_range,
+ *     src/grid_maker.cpp:172; its GPU kernel silently skips, and a kernel
+ *     cannot throw): callers that need the exception check on the host.
+ */
+#ifndef MOLGRID_HIP_H_
+#define MOLGRID_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  MG_OK = 0,
+  MG_ERR_INVALID_ARGUMENT = -1, /* reference: std::invalid_argument */
+  MG_ERR_OUT_OF_RANGE = -2,     /* reference: std::out_of_range */
+  MG_ERR_UNSUPPORTED = -3,
+  MG_ERR_NULL_POINTER = -4
+};
+
+/* Scalar state of a GridMaker; replaces the by-value `GridMaker G` kernel
+ * argument of the reference (src/grid_maker.cu:212-215) and holds the members
+ * declared in include/libmolgrid/grid_maker.h:35-48. */
+typedef struct mg_gridmaker {
+  float resolution;
+  float dimension;
+  float radius_scale;
+  float gaussian_radius_multiple;
+  float final_radius_multiple;
+  float A, B, C; /* quadratic tail of the density */
+  float D, E;    /* its derivative */
+  int32_t binary;
+  int32_t radii_type_indexed;
+  uint32_t dim; /* points per grid side */
+} mg_gridmaker;
+
+/* Host only.  Replaces GridMaker::initialize (src/grid_maker.cpp:15-36) and the
+ * constructor (include/libmolgrid/grid_maker.h:70-74). */
+int mg_gridmaker_init(mg_gridmaker* g, float resolution, float dimension, int binary,
+                      int radii_type_indexed, float radius_scale,
+                      float gaussian_radius_multiple);
+
+/* Human readable text for a return code of this library. */
+const char* mg_error_string(int code);
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mg_version(void);
+
+/* Transform::forward on device coordinates; replaces
+ * transform_forward_kernel + its launcher (src/transform.cu:13-32, 66-75).
+ * out = rotate_q(in - center) + center + translation; `dotranslate` = 0 drops
+ * the translation but still rotates about center.  in == out is allowed. */
+int mg_transform_forward(int nbatch, const int32_t* atom_offsets, int atoms_per_example,
+                         const float* quats, const float quat_host[4],
+                         const float* centers, const float center_host[3],
+                         const float* translations, const float translation_host[3],
+                         int dotranslate, const float* in_coords, float* out_coords,
+                         void* stream);
+
+/* Transform::backward on device coordinates; replaces
+ * transform_translate_kernel / transform_rotate_kernel and their launcher
+ * (src/transform.cu:35-62, 79-93) with the CPU overload's arithmetic
+ * (src/transform.cpp:85-108): out = rotate_{q^-1}(in - translation - center) + center. */
+int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per_example,
+                          const float* quats, const float quat_host[4],
+                          const float* centers, const float center_host[3],
+                          const float* translations, const float translation_host[3],
+                          int dotranslate, const float* in_coords, float* out_coords,
+                          void* stream);
+
+/* GridMaker::forward, index types; replaces forward_gpu and its launcher
+ * (src/grid_maker.cu:212-289) for a whole batch in one launch, with the values
+ * of the CPU overload (src/grid_maker.cpp:153-212).
+ *   coords [n,3], type_index [n], radii [n], out [nbatch, ntypes, dim, dim, dim]
+ * `out` is overwritten completely (no memset needed before the call). */
+int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                     int atoms_per_example, const float* grid_centers,
+                     const float grid_center_host[3], const float* coords,
+                     const float* type_index, const float* radii, int ntypes, float* out,
+                     void* stream);
+
+/* GridMaker::forward, vector types; replaces forward_gpu_vec and its launcher
+ * (src/grid_maker.cu:348-441), values of src/grid_maker.cpp:214-271.
+ *   type_vector [n, ntypes]; radii [n], or [nbatch, ntypes] when
+ *   g->radii_type_indexed. */
+int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                      int atoms_per_example, const float* grid_centers,
+                      const float grid_center_host[3], const float* coords,
+                      const float* type_vector, const float* radii, int ntypes, float* out,
+                      void* stream);
+
+/* GridMaker::backward, index types; replaces set_atom_gradients and its
+ * launcher (src/grid_maker.cu:472-510, 576-595), values of
+ * src/grid_maker.cpp:436-467.
+ *   diff [nbatch, ntypes, dim, dim, dim] -> atom_gradients [n,3] (overwritten;
+ *   ignored atoms get zero). */
+int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                      int atoms_per_example, const float* grid_centers,
+                      const float grid_center_host[3], const float* coords,
+                      const float* type_index, const float* radii, int ntypes,
+                      const float* diff, float* atom_gradients, void* stream);
+
+/* GridMaker::backward, vector types; replaces set_atom_type_gradients and its
+ * launcher (src/grid_maker.cu:513-571, 604-642), values of
+ * src/grid_maker.cpp:477-519.  type_gradients [n, ntypes] is overwritten. */
+int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                       int atoms_per_example, const float* grid_centers,
+                       const float grid_center_host[3], const float* coords,
+                       const float* type_vector, const float* radii, int ntypes,
+                       const float* diff, float* atom_gradients, float* type_gradients,
+                       void* stream);
+
+/* GridInterpolater::forward; replaces gpu_set_outgrid and its per-channel
+ * launch loop (src/grid_interpolater.cu:106-166), values of
+ * src/grid_interpolater.cpp:16-48.  One launch for all examples and channels.
+ *   in  [nbatch, channels, in_dim, in_dim, in_dim]
+ *   out [nbatch, channels, out_dim, out_dim, out_dim], in != out
+ * with in_dim = round(in_dimension/in_resolution)+1 and likewise out_dim. */
+int mg_interpolate(float in_resolution, float in_dimension, float out_resolution,
+                   float out_dimension, int nbatch, int channels,
+                   const float* in_centers, const float in_center_host[3], const float* in,
+                   const float* quats, const float quat_host[4],
+                   const float* rot_centers, const float rot_center_host[3],
+                   const float* translations, const float translation_host[3],
+                   const float* out_centers, const float out_center_host[3], float* out,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOLGRID_HIP_H_ */

@@ -1,0 +1,22 @@
+"""MI355X-native gridding hot path with libmolgrid's interface.
+
+``GridMaker.forward/backward``, ``Transform.forward/backward`` and
+``GridInterpolater.forward`` run as hand-written HIP kernels (gfx950) behind the
+C ABI of ``include/molgrid_hip.h``; this package is the Python host side that
+mirrors the reference's ``molgrid`` module for that path.
+"""
+from ._capi import LIB_PATH, lib as _lib  # noqa: F401  (fails loudly if the .so is missing)
+from .gridding import (CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
+                       float3, set_random_seed, transform_batch)
+
+__version__ = "0.1.0"
+
+
+def get_gpu_device():
+    import torch
+    return torch.cuda.current_device()
+
+
+def set_gpu_device(index):
+    import torch
+    torch.cuda.set_device(int(index))

@@ -1,0 +1,366 @@
+// Atom-gradient (and type-gradient) accumulation on gfx950.
+//
+// One wavefront owns one atom: its 64 lanes sweep the atom's voxel box
+// (src/grid_maker.cu:66-79) in a fixed lane -> voxel order, each lane keeps a
+// private partial sum, and the partials are combined with a DPP reduction tree
+// inside the wave.  No global float atomics are used, so the result is
+// reproducible run to run.  Per-voxel terms follow accumulate_atom_gradient and
+// density_grad_dist (src/grid_maker.cu:881-919); the CPU loops being mirrored
+// are src/grid_maker.cpp:325-389 and 436-519.
+#include "kernels.h"
+#include "splat_common.h"
+
+namespace mg {
+
+namespace {
+
+constexpr int kBwdThreads = 256;
+constexpr int kBwdWaves = kBwdThreads / kWave;
+
+// DPP controls (gfx9 encoding)
+constexpr int kDppQuadPerm1032 = 0xB1;  // quad_perm:[1,0,3,2]
+constexpr int kDppQuadPerm2301 = 0x4E;  // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+constexpr int kDppRowBcast15 = 0x142;
+constexpr int kDppRowBcast31 = 0x143;
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  // lanes outside ROW_MASK (or without a source lane) contribute 0
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+  return v + __int_as_float(moved);
+}
+
+// Sum of v over the 64 lanes of the wave, returned to every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<kDppQuadPerm1032, 0xF>(v);
+  v = dpp_add<kDppQuadPerm2301, 0xF>(v);
+  v = dpp_add<kDppRowHalfMirror, 0xF>(v);
+  v = dpp_add<kDppRowMirror, 0xF>(v);   // every lane of a 16-lane row holds the row total
+  v = dpp_add<kDppRowBcast15, 0xA>(v);  // rows 1 and 3 add the total of rows 0 and 2
+  v = dpp_add<kDppRowBcast31, 0xC>(v);  // rows 2 and 3 add the total of rows 0..1
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// Lane-strided walk over a box of ni*nj*nk voxels, k fastest: lane L visits
+// linear indices L, L+64, L+128, ...  The mixed-radix step of 64 is worked out
+// once per box so that the inner loop needs no division.
+struct BoxWalk {
+  int i, j, k;     // current offset inside the box
+  int di, dj, dk;  // 64 expressed in (nj*nk, nk, 1) digits
+  int nj, nk;
+  __device__ __forceinline__ void start(int lane, int nj_, int nk_) {
+    nj = nj_;
+    nk = nk_;
+    const int plane = nj * nk;
+    i = lane / plane;
+    int r = lane - i * plane;
+    j = r / nk;
+    k = r - j * nk;
+    di = kWave / plane;
+    r = kWave - di * plane;
+    dj = r / nk;
+    dk = r - dj * nk;
+  }
+  __device__ __forceinline__ void next() {
+    k += dk;
+    if (k >= nk) { k -= nk; ++j; }
+    j += dj;
+    if (j >= nj) { j -= nj; ++i; }
+    i += di;
+  }
+};
+
+// d(density)/d(dist) and the scale that turns (voxel - atom) into the
+// gradient term of one voxel: -(1/dist) * agrad_dist * gridval.  Returns 0
+// where the reference skips the voxel (dist == 0 or beyond the cut-off).
+__device__ __forceinline__ float grad_scale(const GridArg& g, float dist2, float inv_ar2,
+                                            float inv_ar, float frm2, float grm2, float gridval) {
+  if (!(dist2 > 0.f)) return 0.f;
+  const float u = dist2 * inv_ar2;
+  if (!(u <= frm2)) return 0.f;
+  const float rinv = __builtin_amdgcn_rsqf(dist2);
+  const float dist = dist2 * rinv;
+  float agd;
+  if (u <= grm2) {
+    agd = -4.0f * dist * inv_ar2 * __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+  } else {
+    agd = (g.D * dist * inv_ar + g.E) * inv_ar;
+  }
+  return -(agd * gridval) * rinv;
+}
+
+template <bool BINARY>
+__device__ __forceinline__ float point_density(const GridArg& g, float dx, float dy, float dz,
+                                               float ar2, float inv_ar2, float frm2, float grm2) {
+  return density<BINARY, false>(g, dx, dy, dz, BINARY ? ar2 : inv_ar2, 0.f, frm2, grm2);
+}
+
+__global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
+    GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
+    const float* __restrict__ type_index, const float* __restrict__ radii,
+    const float* __restrict__ diff, float* __restrict__ atom_gradients) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int b = blockIdx.y;
+  int begin, end;
+  example_range(batch, b, begin, end);
+  const float3 center = load3(centers, b);
+  const float ox = center.x - g.half_dimension;
+  const float oy = center.y - g.half_dimension;
+  const float oz = center.z - g.half_dimension;
+  const int dim = g.dim;
+  const size_t chan_stride = (size_t)dim * dim * dim;
+  const float* diff_b = diff + (size_t)b * g.ntypes * chan_stride;
+  const float frm2 = g.frm * g.frm, grm2 = g.grm * g.grm;
+
+  for (int a = begin + blockIdx.x * kBwdWaves + wave; a < end; a += gridDim.x * kBwdWaves) {
+    float gx = 0.f, gy = 0.f, gz = 0.f;
+    const float tf = roundf(type_index[a]);  // backward rounds, forward floors
+    if (tf >= 0.f && tf < (float)g.ntypes) {
+      const float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
+      const float radius = radii[a];
+      float densityrad, ar;
+      {
+#pragma clang fp contract(off)
+        densityrad = radius * g.radius_scale * g.frm;
+        ar = radius * g.radius_scale;
+      }
+      const float inv_ar = 1.0f / ar;
+      const float inv_ar2 = inv_ar * inv_ar;
+      int lo0, hi0, lo1, hi1, lo2, hi2;
+      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
+      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
+      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
+      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
+      if (ni > 0 && nj > 0 && nk > 0) {
+        const float* chan = diff_b + (size_t)(int)tf * chan_stride;
+        BoxWalk w;
+        w.start(lane, nj, nk);
+        for (; w.i < ni; w.next()) {
+          const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
+          const float dx = grid_coord(ox, xi, g.resolution) - ax;
+          const float dy = grid_coord(oy, yi, g.resolution) - ay;
+          const float dz = grid_coord(oz, zi, g.resolution) - az;
+          const float dist2 = dx * dx + dy * dy + dz * dz;
+          const float gv = chan[((size_t)xi * dim + yi) * dim + zi];
+          const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, gv);
+          gx = fmaf(dx, sc, gx);
+          gy = fmaf(dy, sc, gy);
+          gz = fmaf(dz, sc, gz);
+        }
+      }
+    }
+    gx = wave_sum(gx);
+    gy = wave_sum(gy);
+    gz = wave_sum(gz);
+    if (lane == 0) {
+      atom_gradients[3 * a] = gx;
+      atom_gradients[3 * a + 1] = gy;
+      atom_gradients[3 * a + 2] = gz;
+    }
+  }
+}
+
+// Vector types.  TG channels are handled per pass so that the per-lane type
+// gradient partials stay in registers.
+template <bool BINARY, bool RTI, int TG>
+__global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
+    GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
+    const float* __restrict__ type_vector, const float* __restrict__ radii,
+    const float* __restrict__ diff, float* __restrict__ atom_gradients,
+    float* __restrict__ type_gradients) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int b = blockIdx.y;
+  int begin, end;
+  example_range(batch, b, begin, end);
+  const float3 center = load3(centers, b);
+  const float ox = center.x - g.half_dimension;
+  const float oy = center.y - g.half_dimension;
+  const float oz = center.z - g.half_dimension;
+  const int dim = g.dim;
+  const int T = g.ntypes;
+  const size_t chan_stride = (size_t)dim * dim * dim;
+  const float* diff_b = diff + (size_t)b * T * chan_stride;
+  const float* radii_b = RTI ? radii + (size_t)b * T : radii;
+  const float frm2 = g.frm * g.frm, grm2 = g.grm * g.grm;
+
+  for (int a0 = begin + blockIdx.x * kBwdWaves + wave; a0 < end; a0 += gridDim.x * kBwdWaves) {
+    const int a = __builtin_amdgcn_readfirstlane(a0);
+    const float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
+    const float* __restrict__ tv = type_vector + (size_t)a * T;
+    float gx = 0.f, gy = 0.f, gz = 0.f;
+
+    if (!RTI) {
+      const float radius = radii_b[a];
+      float densityrad, ar, ar2;
+      {
+#pragma clang fp contract(off)
+        densityrad = radius * g.radius_scale * g.frm;
+        ar = radius * g.radius_scale;
+        ar2 = ar * ar;
+      }
+      const float inv_ar = 1.0f / ar;
+      const float inv_ar2 = inv_ar * inv_ar;
+      int lo0, hi0, lo1, hi1, lo2, hi2;
+      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
+      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
+      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
+      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
+      const bool any = ni > 0 && nj > 0 && nk > 0;
+      for (int cbase = 0; cbase < T; cbase += TG) {
+        const int nchan = min(TG, T - cbase);
+        float tg[TG];
+#pragma unroll
+        for (int t = 0; t < TG; ++t) tg[t] = 0.f;
+        if (any) {
+          BoxWalk w;
+          w.start(lane, nj, nk);
+          for (; w.i < ni; w.next()) {
+            const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
+            const float dx = grid_coord(ox, xi, g.resolution) - ax;
+            const float dy = grid_coord(oy, yi, g.resolution) - ay;
+            const float dz = grid_coord(oz, zi, g.resolution) - az;
+            const float dist2 = dx * dx + dy * dy + dz * dz;
+            const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+            const float* p = diff_b + (size_t)cbase * chan_stride + ((size_t)xi * dim + yi) * dim + zi;
+            float weighted = 0.f;  // sum_t weight_t * diff_t at this voxel
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+              if (t < nchan) {
+                const float gv = p[(size_t)t * chan_stride];
+                tg[t] = fmaf(val, gv, tg[t]);
+                weighted = fmaf(tv[cbase + t], gv, weighted);
+              }
+            }
+            const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, weighted);
+            gx = fmaf(dx, sc, gx);
+            gy = fmaf(dy, sc, gy);
+            gz = fmaf(dz, sc, gz);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+          if (t < nchan) {
+            const float s = wave_sum(tg[t]);
+            if (lane == 0) type_gradients[(size_t)a * T + cbase + t] = s;
+          }
+        }
+      }
+    } else {
+      // radius per type: every channel has its own box
+      for (int t = 0; t < T; ++t) {
+        const float radius = radii_b[t];
+        const float tm = tv[t];
+        float densityrad, ar, ar2;
+        {
+#pragma clang fp contract(off)
+          densityrad = radius * g.radius_scale * g.frm;
+          ar = radius * g.radius_scale;
+          ar2 = ar * ar;
+        }
+        const float inv_ar = 1.0f / ar;
+        const float inv_ar2 = inv_ar * inv_ar;
+        int lo0, hi0, lo1, hi1, lo2, hi2;
+        bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
+        bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
+        bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
+        const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
+        float tgt = 0.f, tx = 0.f, ty = 0.f, tz = 0.f;
+        if (ni > 0 && nj > 0 && nk > 0) {
+          const float* chan = diff_b + (size_t)t * chan_stride;
+          BoxWalk w;
+          w.start(lane, nj, nk);
+          for (; w.i < ni; w.next()) {
+            const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
+            const float dx = grid_coord(ox, xi, g.resolution) - ax;
+            const float dy = grid_coord(oy, yi, g.resolution) - ay;
+            const float dz = grid_coord(oz, zi, g.resolution) - az;
+            const float dist2 = dx * dx + dy * dy + dz * dz;
+            const float gv = chan[((size_t)xi * dim + yi) * dim + zi];
+            const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+            tgt = fmaf(val, gv, tgt);
+            const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, gv);
+            tx = fmaf(dx, sc, tx);
+            ty = fmaf(dy, sc, ty);
+            tz = fmaf(dz, sc, tz);
+          }
+        }
+        const float s = wave_sum(tgt);
+        if (lane == 0) type_gradients[(size_t)a * T + t] = s;
+        if (tm != 0.f) {
+          gx = fmaf(tx, tm, gx);
+          gy = fmaf(ty, tm, gy);
+          gz = fmaf(tz, tm, gz);
+        }
+      }
+    }
+    gx = wave_sum(gx);
+    gy = wave_sum(gy);
+    gz = wave_sum(gz);
+    if (lane == 0) {
+      atom_gradients[3 * a] = gx;
+      atom_gradients[3 * a + 1] = gy;
+      atom_gradients[3 * a + 2] = gz;
+    }
+  }
+}
+
+int backward_blocks(int launch_atoms) {
+  int blocks = (launch_atoms + kBwdWaves - 1) / kBwdWaves;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  return blocks;
+}
+
+template <bool BINARY, bool RTI>
+hipError_t launch_vec(const GridArg& g, const BatchArg& batch, int nbatch, int launch_atoms,
+                      const Vec3Arg& centers, const float* coords, const float* type_vector,
+                      const float* radii, const float* diff, float* atom_gradients,
+                      float* type_gradients, hipStream_t stream) {
+  dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
+  if (g.ntypes <= 8)
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 8>), grid, block, 0, stream, g, batch,
+                       centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
+  else if (g.ntypes <= 16)
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 16>), grid, block, 0, stream, g, batch,
+                       centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
+  else
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 32>), grid, block, 0, stream, g, batch,
+                       centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 int launch_atoms, const Vec3Arg& centers, const float* coords,
+                                 const float* type_index, const float* radii, const float* diff,
+                                 float* atom_gradients, hipStream_t stream) {
+  dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
+  hipLaunchKernelGGL(backward_index_kernel, grid, block, 0, stream, g, batch, centers, coords,
+                     type_index, radii, diff, atom_gradients);
+  return hipGetLastError();
+}
+
+hipError_t launch_backward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
+                                  int launch_atoms, const Vec3Arg& centers, const float* coords,
+                                  const float* type_vector, const float* radii, const float* diff,
+                                  float* atom_gradients, float* type_gradients, bool binary,
+                                  bool radii_type_indexed, hipStream_t stream) {
+  if (binary && radii_type_indexed)
+    return launch_vec<true, true>(g, batch, nbatch, launch_atoms, centers, coords, type_vector,
+                                  radii, diff, atom_gradients, type_gradients, stream);
+  if (binary)
+    return launch_vec<true, false>(g, batch, nbatch, launch_atoms, centers, coords, type_vector,
+                                   radii, diff, atom_gradients, type_gradients, stream);
+  if (radii_type_indexed)
+    return launch_vec<false, true>(g, batch, nbatch, launch_atoms, centers, coords, type_vector,
+                                   radii, diff, atom_gradients, type_gradients, stream);
+  return launch_vec<false, false>(g, batch, nbatch, launch_atoms, centers, coords, type_vector,
+                                  radii, diff, atom_gradients, type_gradients, stream);
+}
+
+}  // namespace mg

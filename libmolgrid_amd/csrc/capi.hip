@@ -1,0 +1,266 @@
+// C ABI of the gridding library: argument checks, then one kernel launch per
+// call on the caller's stream.  Nothing here allocates or synchronises.
+#include <cmath>
+#include <cstring>
+
+#include "kernels.h"
+#include "molgrid_hip.h"
+
+namespace {
+
+using namespace mg;
+
+Vec3Arg vec3(const float* dev, const float* host) {
+  Vec3Arg v;
+  v.dev = dev;
+  for (int i = 0; i < 3; ++i) v.host[i] = (dev == nullptr && host != nullptr) ? host[i] : 0.f;
+  return v;
+}
+
+Vec4Arg vec4(const float* dev, const float* host) {
+  Vec4Arg v;
+  v.dev = dev;
+  // identity rotation when nothing is given
+  v.host[0] = 1.f;
+  v.host[1] = v.host[2] = v.host[3] = 0.f;
+  if (dev == nullptr && host != nullptr)
+    for (int i = 0; i < 4; ++i) v.host[i] = host[i];
+  return v;
+}
+
+GridArg grid_arg(const mg_gridmaker* g, int ntypes) {
+  GridArg a;
+  a.resolution = g->resolution;
+  a.half_dimension = (float)(g->dimension / 2.0);  // src/grid_maker.cpp:101
+  a.radius_scale = g->radius_scale;
+  a.grm = g->gaussian_radius_multiple;
+  a.frm = g->final_radius_multiple;
+  a.A = g->A;
+  a.B = g->B;
+  a.C = g->C;
+  a.D = g->D;
+  a.E = g->E;
+  a.dim = (int)g->dim;
+  a.ntypes = ntypes;
+  return a;
+}
+
+// The fast kernels test the cut-offs on (dist/ar)^2 and do not clip to the
+// per-atom index box.  That is indistinguishable from the reference when the
+// density reaches zero at the cut-off and the box is wider than the support.
+// A truncated Gaussian (negative gaussian_radius_multiple at construction:
+// no quadratic tail, final == gaussian multiple) or a binary sphere wider than
+// the box need the reference's exact predicates.
+bool needs_exact(const mg_gridmaker* g) {
+  if (g->binary) return g->final_radius_multiple < 1.0f;
+  return g->final_radius_multiple <= g->gaussian_radius_multiple;
+}
+
+int check_common(const mg_gridmaker* g, int nbatch, const int32_t* offsets, int per_example,
+                 int ntypes) {
+  if (g == nullptr) return MG_ERR_NULL_POINTER;
+  if (nbatch < 0 || ntypes < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (offsets == nullptr && per_example < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (g->dim == 0 || g->dim > 65535u) return MG_ERR_OUT_OF_RANGE;
+  if (!(g->resolution > 0.f)) return MG_ERR_INVALID_ARGUMENT;
+  return MG_OK;
+}
+
+int from_hip(hipError_t e) { return e == hipSuccess ? MG_OK : (int)e; }
+
+}  // namespace
+
+extern "C" {
+
+int mg_version(void) { return 100; }
+
+const char* mg_error_string(int code) {
+  switch (code) {
+    case MG_OK: return "success";
+    case MG_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case MG_ERR_OUT_OF_RANGE: return "argument out of range";
+    case MG_ERR_UNSUPPORTED: return "unsupported configuration";
+    case MG_ERR_NULL_POINTER: return "required pointer is null";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown error";
+}
+
+int mg_gridmaker_init(mg_gridmaker* g, float resolution, float dimension, int binary,
+                      int radii_type_indexed, float radius_scale, float grm) {
+  if (g == nullptr) return MG_ERR_NULL_POINTER;
+  std::memset(g, 0, sizeof(*g));
+  g->resolution = resolution;
+  g->dimension = dimension;
+  g->radius_scale = radius_scale;
+  g->binary = binary ? 1 : 0;
+  g->radii_type_indexed = radii_type_indexed ? 1 : 0;
+  // A negative multiple asks for a Gaussian truncated at |grm| with no
+  // quadratic tail; otherwise the tail ends at (1 + 2 grm^2) / (2 grm).
+  if (grm < 0) {
+    g->gaussian_radius_multiple = -grm;
+    g->final_radius_multiple = -grm;
+  } else {
+    g->gaussian_radius_multiple = grm;
+    g->final_radius_multiple = (1 + 2 * grm * grm) / (2 * grm);
+  }
+  g->dim = (uint32_t)(std::round(dimension / resolution) + 1);
+  // Quadratic a*(d/r)^2 + b*(d/r) + c matching value and slope of the Gaussian
+  // at d = grm*r and reaching zero with zero slope at the final multiple; the
+  // exponential is taken in double and the results are stored as float.
+  const double e = std::exp((double)(-2 * grm * grm));
+  g->A = (float)(e * 4 * grm * grm);
+  g->B = (float)(-e * (4 * grm + 8 * grm * grm * grm));
+  g->C = (float)(e * (4 * grm * grm * grm * grm + 4 * grm * grm + 1));
+  g->D = (float)(8 * grm * grm * std::exp(-2.0 * grm * grm));
+  g->E = (float)(-(4 * grm + 8 * grm * grm * grm) * e);
+  return MG_OK;
+}
+
+int mg_transform_forward(int nbatch, const int32_t* atom_offsets, int atoms_per_example,
+                         const float* quats, const float quat_host[4], const float* centers,
+                         const float center_host[3], const float* translations,
+                         const float translation_host[3], int dotranslate,
+                         const float* in_coords, float* out_coords, void* stream) {
+  if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
+    return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (in_coords == nullptr || out_coords == nullptr) return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_transform(batch, nbatch, atoms_per_example, vec4(quats, quat_host),
+                                   vec3(centers, center_host),
+                                   vec3(translations, translation_host), dotranslate != 0, false,
+                                   in_coords, out_coords, (hipStream_t)stream));
+}
+
+int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per_example,
+                          const float* quats, const float quat_host[4], const float* centers,
+                          const float center_host[3], const float* translations,
+                          const float translation_host[3], int dotranslate,
+                          const float* in_coords, float* out_coords, void* stream) {
+  if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
+    return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (in_coords == nullptr || out_coords == nullptr) return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_transform(batch, nbatch, atoms_per_example, vec4(quats, quat_host),
+                                   vec3(centers, center_host),
+                                   vec3(translations, translation_host), dotranslate != 0, true,
+                                   in_coords, out_coords, (hipStream_t)stream));
+}
+
+int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                     int atoms_per_example, const float* grid_centers,
+                     const float grid_center_host[3], const float* coords,
+                     const float* type_index, const float* radii, int ntypes, float* out,
+                     void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  // src/grid_maker.cpp:160-162
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || ntypes == 0) return MG_OK;
+  if (out == nullptr) return MG_ERR_NULL_POINTER;
+  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
+  if (has_atoms && (coords == nullptr || type_index == nullptr || radii == nullptr))
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_forward_index(grid_arg(g, ntypes), batch, nbatch,
+                                       vec3(grid_centers, grid_center_host), coords, type_index,
+                                       radii, out, g->binary != 0, needs_exact(g),
+                                       (hipStream_t)stream));
+}
+
+int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                      int atoms_per_example, const float* grid_centers,
+                      const float grid_center_host[3], const float* coords,
+                      const float* type_vector, const float* radii, int ntypes, float* out,
+                      void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  if (nbatch == 0 || ntypes == 0) return MG_OK;
+  if (out == nullptr) return MG_ERR_NULL_POINTER;
+  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
+  if (has_atoms && (coords == nullptr || type_vector == nullptr || radii == nullptr))
+    return MG_ERR_NULL_POINTER;
+  if (g->radii_type_indexed && radii == nullptr) return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_forward_vector(grid_arg(g, ntypes), batch, nbatch,
+                                        vec3(grid_centers, grid_center_host), coords,
+                                        type_vector, radii, out, g->binary != 0,
+                                        g->radii_type_indexed != 0, needs_exact(g),
+                                        (hipStream_t)stream));
+}
+
+int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                      int atoms_per_example, const float* grid_centers,
+                      const float grid_center_host[3], const float* coords,
+                      const float* type_index, const float* radii, int ntypes,
+                      const float* diff, float* atom_gradients, void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  // src/grid_maker.cpp:442-444
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (coords == nullptr || type_index == nullptr || radii == nullptr || diff == nullptr ||
+      atom_gradients == nullptr)
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_backward_index(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
+                                        vec3(grid_centers, grid_center_host), coords,
+                                        type_index, radii, diff, atom_gradients,
+                                        (hipStream_t)stream));
+}
+
+int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                       int atoms_per_example, const float* grid_centers,
+                       const float grid_center_host[3], const float* coords,
+                       const float* type_vector, const float* radii, int ntypes,
+                       const float* diff, float* atom_gradients, float* type_gradients,
+                       void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (coords == nullptr || type_vector == nullptr || radii == nullptr || diff == nullptr ||
+      atom_gradients == nullptr || type_gradients == nullptr)
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_backward_vector(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
+                                         vec3(grid_centers, grid_center_host), coords,
+                                         type_vector, radii, diff, atom_gradients,
+                                         type_gradients, g->binary != 0,
+                                         g->radii_type_indexed != 0, (hipStream_t)stream));
+}
+
+int mg_interpolate(float in_resolution, float in_dimension, float out_resolution,
+                   float out_dimension, int nbatch, int channels, const float* in_centers,
+                   const float in_center_host[3], const float* in, const float* quats,
+                   const float quat_host[4], const float* rot_centers,
+                   const float rot_center_host[3], const float* translations,
+                   const float translation_host[3], const float* out_centers,
+                   const float out_center_host[3], float* out, void* stream) {
+  if (nbatch < 0 || channels < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (!(in_resolution > 0.f) || !(out_resolution > 0.f)) return MG_ERR_INVALID_ARGUMENT;
+  // src/grid_interpolater.cpp:58-60, 70-75
+  if (in == nullptr || out == nullptr) return MG_ERR_INVALID_ARGUMENT;
+  if (in == out) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || channels == 0) return MG_OK;
+  InterpArg p;
+  p.in_resolution = in_resolution;
+  p.out_resolution = out_resolution;
+  p.in_half = (float)(in_dimension / 2.0);
+  p.out_half = (float)(out_dimension / 2.0);
+  // include/libmolgrid/grid_interpolater.h:59-64
+  p.in_dim = (int)(std::round(in_dimension / in_resolution) + 1);
+  p.out_dim = (int)(std::round(out_dimension / out_resolution) + 1);
+  p.channels = channels;
+  if (p.in_dim <= 0 || p.out_dim <= 0 || p.in_dim > 1200 || p.out_dim > 1200)
+    return MG_ERR_OUT_OF_RANGE;
+  return from_hip(launch_interpolate(p, nbatch, vec3(in_centers, in_center_host), in,
+                                     vec4(quats, quat_host), vec3(rot_centers, rot_center_host),
+                                     vec3(translations, translation_host),
+                                     vec3(out_centers, out_center_host), out,
+                                     (hipStream_t)stream));
+}
+
+}  // extern "C"

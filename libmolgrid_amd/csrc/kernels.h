@@ -1,0 +1,58 @@
+// Host-callable launchers of the gfx950 kernels (internal to the library; the
+// public surface is the C ABI in include/molgrid_hip.h).
+#ifndef LIBMOLGRID_AMD_KERNELS_H_
+#define LIBMOLGRID_AMD_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+
+namespace mg {
+
+// Channels whose accumulators one workgroup keeps in LDS at a time
+// (32 * 512 voxels * 4 B = 64 KiB); grids with more channels take several
+// passes over the atom list.
+constexpr int kMaxChannelGroup = 32;
+
+struct InterpArg {
+  float in_resolution, out_resolution;
+  float in_half, out_half;  // (float)(dimension / 2.0)
+  int in_dim, out_dim;
+  int channels;
+};
+
+hipError_t launch_transform(const BatchArg& batch, int nbatch, int launch_atoms,
+                            const Vec4Arg& quats, const Vec3Arg& centers,
+                            const Vec3Arg& translations, bool dotranslate, bool inverse,
+                            const float* in, float* out, hipStream_t stream);
+
+hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nbatch,
+                                const Vec3Arg& centers, const float* coords,
+                                const float* type_index, const float* radii, float* out,
+                                bool binary, bool exact, hipStream_t stream);
+
+hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 const Vec3Arg& centers, const float* coords,
+                                 const float* type_vector, const float* radii, float* out,
+                                 bool binary, bool radii_type_indexed, bool exact,
+                                 hipStream_t stream);
+
+hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 int launch_atoms, const Vec3Arg& centers, const float* coords,
+                                 const float* type_index, const float* radii, const float* diff,
+                                 float* atom_gradients, hipStream_t stream);
+
+hipError_t launch_backward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
+                                  int launch_atoms, const Vec3Arg& centers, const float* coords,
+                                  const float* type_vector, const float* radii, const float* diff,
+                                  float* atom_gradients, float* type_gradients, bool binary,
+                                  bool radii_type_indexed, hipStream_t stream);
+
+hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_centers,
+                              const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
+                              const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,
+                              hipStream_t stream);
+
+}  // namespace mg
+
+#endif

@@ -1,0 +1,941 @@
+"""Host-side mirror of libmolgrid's gridding classes on top of the HIP C ABI.
+
+``GridMaker``, ``GridInterpolater``, ``Transform``, ``Quaternion``, ``float3`` and
+``CoordinateSet`` keep the names, argument order and error behaviour of the
+reference's Python module (python/bindings.in.cpp:286-309, 455-520, 816-943)
+for the gridding path.  Every numeric call validates its arguments as the
+reference does (std::out_of_range -> IndexError, std::invalid_argument ->
+ValueError) and then makes exactly one call into ``libmolgrid_hip.so``.
+
+Arrays may be ROCm torch tensors (used in place, on torch's current stream) or
+host arrays (numpy / CPU tensors): host arrays are staged through device memory
+and the kernels still do the work -- there is no CPU implementation here.
+"""
+import math
+
+import numpy as np
+import torch
+
+from . import _capi
+
+_lib = _capi.lib
+
+
+# --------------------------------------------------------------------------- #
+# small value types
+# --------------------------------------------------------------------------- #
+class float3(object):
+    """x, y, z triple; any 3-sequence converts (bindings.in.cpp:286-309)."""
+    __slots__ = ("x", "y", "z")
+
+    def __init__(self, x=0.0, y=0.0, z=0.0):
+        self.x, self.y, self.z = float(x), float(y), float(z)
+
+    def __iter__(self):
+        return iter((self.x, self.y, self.z))
+
+    def __len__(self):
+        return 3
+
+    def __getitem__(self, i):
+        return (self.x, self.y, self.z)[i]
+
+    def __eq__(self, o):
+        return tuple(self) == tuple(o)
+
+    def __repr__(self):
+        return "float3(%g, %g, %g)" % (self.x, self.y, self.z)
+
+
+def _to_float3(v):
+    if isinstance(v, float3):
+        return v
+    if isinstance(v, torch.Tensor):
+        v = v.detach().cpu().tolist()
+    v = tuple(v)
+    if len(v) != 3:
+        raise ValueError("expected a sequence of 3 floats")
+    return float3(*v)
+
+
+_f32 = np.float32
+
+
+class Quaternion(object):
+    """Single-precision quaternion (a + bi + cj + dk), not assumed normalised.
+
+    Arithmetic is done in float32 in the association order of
+    include/libmolgrid/quaternion.h:82-166 so that host-side results are the
+    same floats the device kernels produce.
+    """
+    __slots__ = ("a", "b", "c", "d")
+
+    def __init__(self, a=1.0, b=0.0, c=0.0, d=0.0):
+        self.a, self.b, self.c, self.d = _f32(a), _f32(b), _f32(c), _f32(d)
+
+    def R_component_1(self):
+        return float(self.a)
+
+    def R_component_2(self):
+        return float(self.b)
+
+    def R_component_3(self):
+        return float(self.c)
+
+    def R_component_4(self):
+        return float(self.d)
+
+    def real(self):
+        return float(self.a)
+
+    def as_tuple(self):
+        return (float(self.a), float(self.b), float(self.c), float(self.d))
+
+    def __eq__(self, o):
+        return isinstance(o, Quaternion) and self.as_tuple() == o.as_tuple()
+
+    def __repr__(self):
+        return "Quaternion(%g, %g, %g, %g)" % self.as_tuple()
+
+    def __mul__(self, r):
+        if not isinstance(r, Quaternion):
+            r = _f32(r)
+            return Quaternion(self.a * r, self.b * r, self.c * r, self.d * r)
+        a, b, c, d = self.a, self.b, self.c, self.d
+        return Quaternion(+a * r.a - b * r.b - c * r.c - d * r.d,
+                          +a * r.b + b * r.a + c * r.d - d * r.c,
+                          +a * r.c - b * r.d + c * r.a + d * r.b,
+                          +a * r.d + b * r.c - c * r.b + d * r.a)
+
+    def __truediv__(self, r):
+        if not isinstance(r, Quaternion):
+            r = _f32(r)
+            return Quaternion(self.a / r, self.b / r, self.c / r, self.d / r)
+        a, b, c, d = self.a, self.b, self.c, self.d
+        den = r.a * r.a + r.b * r.b + r.c * r.c + r.d * r.d
+        return Quaternion((+a * r.a + b * r.b + c * r.c + d * r.d) / den,
+                          (-a * r.b + b * r.a - c * r.d + d * r.c) / den,
+                          (-a * r.c + b * r.d + c * r.a - d * r.b) / den,
+                          (-a * r.d - b * r.c + c * r.b + d * r.a) / den)
+
+    def conj(self):
+        return Quaternion(self.a, -self.b, -self.c, -self.d)
+
+    def norm(self):
+        """Cayley norm: the square of the Euclidean length."""
+        return float(self.a * self.a + self.b * self.b + self.c * self.c + self.d * self.d)
+
+    def inverse(self):
+        n = self.a * self.a + self.b * self.b + self.c * self.c + self.d * self.d
+        return Quaternion(self.a / n, -self.b / n, -self.c / n, -self.d / n)
+
+    def rotate(self, x, y, z):
+        p = self * Quaternion(0, x, y, z) * (self.conj() / _f32(self.norm()))
+        return float3(p.b, p.c, p.d)
+
+    def transform(self, x, y, z, center, translate):
+        center, translate = _to_float3(center), _to_float3(translate)
+        pt = self.rotate(_f32(x) - _f32(center.x), _f32(y) - _f32(center.y),
+                         _f32(z) - _f32(center.z))
+        return float3(_f32(pt.x) + _f32(center.x) + _f32(translate.x),
+                      _f32(pt.y) + _f32(center.y) + _f32(translate.y),
+                      _f32(pt.z) + _f32(center.z) + _f32(translate.z))
+
+
+# random source for Transform's random constructor (the reference keeps one
+# global engine, src/libmolgrid.cpp:11; set_random_seed reseeds it)
+_rng = np.random.default_rng()
+
+
+def set_random_seed(seed):
+    global _rng
+    _rng = np.random.default_rng(int(seed))
+
+
+# --------------------------------------------------------------------------- #
+# array staging
+# --------------------------------------------------------------------------- #
+def _device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("libmolgrid_amd needs a ROCm device: the gridding kernels have no "
+                           "CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+class _Arg(object):
+    """A user array made visible to the device.
+
+    ROCm tensors are used in place after the checks of
+    python/bindings_grids.cpp:91-137 (float32, contiguous, on the current
+    device).  Host arrays are copied to the device when the pointer is first
+    asked for (after all shape checks have passed) and, for outputs, back.
+    """
+
+    def __init__(self, x, name, ndim, out=False):
+        self.name = name
+        self.out = out
+        self.host = None
+        self.t = None
+        if isinstance(x, torch.Tensor) and x.is_cuda:
+            if x.dtype != torch.float32:
+                raise ValueError("%s: only float32 device tensors are supported" % name)
+            if not x.is_contiguous():
+                raise ValueError("%s: tensor is not contiguous" % name)
+            if x.device.index != torch.cuda.current_device():
+                raise ValueError("%s: tensor is on device %d but the current device is %d"
+                                 % (name, x.device.index, torch.cuda.current_device()))
+            self.t = x
+            self.shape = tuple(x.shape)
+        else:
+            if isinstance(x, torch.Tensor):
+                if x.dtype != torch.float32:
+                    raise ValueError("%s: only float32 tensors are supported" % name)
+                if not x.is_contiguous():
+                    raise ValueError("%s: tensor is not contiguous" % name)
+                self.host = x.detach()
+            elif out:
+                if not (isinstance(x, np.ndarray) and x.dtype == np.float32
+                        and x.flags.c_contiguous and x.flags.writeable):
+                    raise ValueError("%s: output must be a writable C-contiguous float32 "
+                                     "array" % name)
+                self.host = torch.from_numpy(x)
+            else:
+                self.host = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32))
+            self.shape = tuple(self.host.shape)
+        if len(self.shape) != ndim:
+            raise ValueError("%s: expected %d dimensions, got %d" % (name, ndim, len(self.shape)))
+
+    @property
+    def ptr(self):
+        if self.t is None:
+            self.t = (torch.empty(self.shape, dtype=torch.float32, device=_device()) if self.out
+                      else self.host.to(_device()))
+        return self.t.data_ptr() if self.t.numel() else None
+
+    def finish(self):
+        if self.out and self.host is not None and self.t is not None:
+            self.host.copy_(self.t)
+
+
+def _same_memory(a, b):
+    try:
+        pa = a.data_ptr() if isinstance(a, torch.Tensor) else a.ctypes.data
+        pb = b.data_ptr() if isinstance(b, torch.Tensor) else b.ctypes.data
+    except AttributeError:
+        return False
+    return pa == pb and pa != 0
+
+
+def _is_host(x):
+    return not (isinstance(x, torch.Tensor) and x.is_cuda)
+
+
+def _small_device(values, width):
+    """B x width float32 parameter rows on the device (None -> None)."""
+    if values is None:
+        return None
+    if isinstance(values, torch.Tensor) and values.is_cuda:
+        t = values
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("per-example parameters must be contiguous float32")
+    else:
+        t = torch.as_tensor(np.ascontiguousarray(values, dtype=np.float32)).to(_device())
+    if t.dim() != 2 or t.shape[1] != width:
+        raise ValueError("per-example parameters must have shape (B, %d)" % width)
+    return t
+
+
+def _offsets_arg(offsets, nbatch_hint=None):
+    """(device int32 tensor, nbatch, largest example) for a ragged batch."""
+    if isinstance(offsets, torch.Tensor) and offsets.is_cuda:
+        if offsets.dtype != torch.int32 or not offsets.is_contiguous() or offsets.dim() != 1:
+            raise ValueError("atom offsets on the device must be contiguous int32")
+        host = offsets.cpu().numpy()
+        dev = offsets
+    else:
+        host = np.ascontiguousarray(offsets, dtype=np.int64)
+        dev = torch.as_tensor(host.astype(np.int32)).to(_device())
+    if host.ndim != 1 or host.size < 1:
+        raise ValueError("atom offsets must be a 1-D array of length batch+1")
+    if np.any(np.diff(host) < 0) or host[0] < 0:
+        raise ValueError("atom offsets must be non-decreasing")
+    largest = int(np.max(np.diff(host))) if host.size > 1 else 0
+    return dev, host.size - 1, max(largest, 1), int(host[-1])
+
+
+_Z3 = (0.0, 0.0, 0.0)
+_IDQ = (1.0, 0.0, 0.0, 0.0)
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None and t.numel() else None
+
+
+# --------------------------------------------------------------------------- #
+# Transform
+# --------------------------------------------------------------------------- #
+class Transform(object):
+    """Rigid transform: rotate about ``center`` by ``Q``, then translate.
+
+    Constructors (include/libmolgrid/transform.h:33-55):
+      Transform()                                   identity
+      Transform(Q, center=(0,0,0), translate=(0,0,0))
+      Transform(center, random_translate=0.0, random_rotate=False)
+    The random constructor draws the translation first (three U(-1,1) values
+    scaled by ``random_translate``) and then a uniform rotation from three unit
+    samples (src/transform.cpp:13-33).
+    """
+
+    def __init__(self, *args, **kw):
+        self.Q = Quaternion()
+        self.center = float3()
+        self.translate = float3()
+        if not args and not kw:
+            return
+        first = args[0] if args else kw.get("Q", kw.get("center"))
+        if isinstance(first, Quaternion):
+            names = ("Q", "center", "translate")
+            vals = dict(zip(names, args))
+            vals.update(kw)
+            self.Q = vals["Q"]
+            self.center = _to_float3(vals.get("center", _Z3))
+            self.translate = _to_float3(vals.get("translate", _Z3))
+        else:
+            names = ("center", "random_translate", "random_rotate")
+            vals = dict(zip(names, args))
+            vals.update(kw)
+            self.center = _to_float3(vals["center"])
+            rt = float(vals.get("random_translate", 0.0))
+            r = _rng.uniform(-1.0, 1.0, 3)
+            self.translate = float3(_f32(r[0] * rt), _f32(r[1] * rt), _f32(r[2] * rt))
+            if vals.get("random_rotate", False):
+                u1, u2, u3 = _rng.uniform(0.0, 1.0, 3)
+                sq1, sqr = math.sqrt(1 - u1), math.sqrt(u1)
+                self.Q = Quaternion(sq1 * math.sin(2 * math.pi * u2),
+                                    sq1 * math.cos(2 * math.pi * u2),
+                                    sqr * math.sin(2 * math.pi * u3),
+                                    sqr * math.cos(2 * math.pi * u3))
+
+    def get_quaternion(self):
+        return self.Q
+
+    def get_rotation_center(self):
+        return self.center
+
+    def get_translation(self):
+        return self.translate
+
+    def set_quaternion(self, q):
+        self.Q = q
+
+    def set_rotation_center(self, c):
+        self.center = _to_float3(c)
+
+    def set_translation(self, t):
+        self.translate = _to_float3(t)
+
+    def is_identity(self):
+        return self.Q == Quaternion() and tuple(self.translate) == _Z3
+
+    def _apply(self, fn, what, src, dst, dotranslate):
+        if isinstance(src, CoordinateSet):
+            if not isinstance(dst, CoordinateSet):
+                raise ValueError("output must be a CoordinateSet as well")
+            if src.coords.shape[0] != dst.coords.shape[0]:
+                raise ValueError("Incompatible coordinateset sizes")
+            src, dst = src.coords, dst.coords
+        same = dst is src
+        a_in = _Arg(src, "in", 2)
+        a_out = a_in if same and not _is_host(src) else _Arg(dst, "out", 2, out=True)
+        # transform.h:131-146 (checkGrids)
+        if a_in.shape[0] != a_out.shape[0]:
+            raise ValueError("Different dimensions and input and output coordinates grids.")
+        if a_in.shape[1] != 3:
+            raise ValueError("Input coordinates wrong dimension.")
+        if a_out.shape[1] != 3:
+            raise ValueError("Output coordinates are wrong dimension.")
+        n = a_in.shape[0]
+        code = fn(1, None, n, None, _capi.f4(self.Q.as_tuple()), None, _capi.f3(self.center),
+                  None, _capi.f3(self.translate), int(bool(dotranslate)), a_in.ptr, a_out.ptr,
+                  _stream())
+        _capi.check(code, what)
+        a_out.finish()
+
+    def forward(self, src, dst, dotranslate=True):
+        """dst = Q.rotate(src - center) + center (+ translate).  In place is fine."""
+        self._apply(_lib.mg_transform_forward, "Transform.forward", src, dst, dotranslate)
+
+    def backward(self, src, dst, dotranslate=True):
+        """Inverse: un-translate, then rotate by the inverse about center."""
+        self._apply(_lib.mg_transform_backward, "Transform.backward", src, dst, dotranslate)
+
+
+def transform_batch(offsets, quats, centers, translations, src, dst, dotranslate=True,
+                    inverse=False):
+    """Apply one rigid transform per example to a packed (ragged) batch of atoms.
+
+    offsets: batch+1 atom offsets; quats (B,4), centers (B,3), translations (B,3).
+    """
+    off, nbatch, largest, total = _offsets_arg(offsets)
+    q, c, t = _small_device(quats, 4), _small_device(centers, 3), _small_device(translations, 3)
+    a_in = _Arg(src, "in", 2)
+    a_out = a_in if dst is src and not _is_host(src) else _Arg(dst, "out", 2, out=True)
+    if a_in.shape != a_out.shape or a_in.shape[1] != 3 or a_in.shape[0] < total:
+        raise ValueError("coordinate arrays must both be (n, 3) with n >= offsets[-1]")
+    for name, v in (("quats", q), ("centers", c), ("translations", t)):
+        if v is not None and v.shape[0] != nbatch:
+            raise ValueError("Mismatched batch sizes: %s has %d rows vs %d"
+                             % (name, v.shape[0], nbatch))
+    fn = _lib.mg_transform_backward if inverse else _lib.mg_transform_forward
+    code = fn(nbatch, _ptr(off), largest, _ptr(q), _capi.f4(_IDQ), _ptr(c), _capi.f3(_Z3),
+              _ptr(t), _capi.f3(_Z3), int(bool(dotranslate)), a_in.ptr, a_out.ptr, _stream())
+    _capi.check(code, "transform_batch")
+    a_out.finish()
+
+
+# --------------------------------------------------------------------------- #
+# CoordinateSet (array constructors only)
+# --------------------------------------------------------------------------- #
+class CoordinateSet(object):
+    """Atoms of one molecule: coords (N,3), index types (N) or type vectors
+    (N,T), radii (N).  Only the array constructors of
+    include/libmolgrid/coordinateset.h:60-92 exist here; building one from a
+    molecule file needs a chemistry toolkit and is outside the gridding path.
+    """
+
+    def __init__(self, coords, types, radii, max_type=None):
+        self.coords = coords
+        self.radii = radii
+        tshape = tuple(types.shape)
+        if len(tshape) == 1:
+            if max_type is None:
+                raise ValueError("max_type is required with index types")
+            self.type_index, self.type_vector = types, None
+            self.max_type = int(max_type)
+        elif len(tshape) == 2:
+            self.type_index, self.type_vector = None, types
+            self.max_type = tshape[1]
+        else:
+            raise ValueError("types must be 1-D (indices) or 2-D (vectors)")
+        n = tuple(coords.shape)[0]
+        if tshape[0] != n:
+            raise ValueError("Types and coordinates are of different sizes")
+        if tuple(radii.shape)[0] != n and len(tshape) == 1:
+            raise ValueError("Radii and coordinates are of different sizes")
+
+    def has_indexed_types(self):
+        return self.type_index is not None
+
+    def has_vector_types(self):
+        return self.type_vector is not None
+
+    def size(self):
+        return tuple(self.coords.shape)[0]
+
+    def __len__(self):
+        return self.size()
+
+    def num_types(self):
+        return self.max_type
+
+    def center(self):
+        """Mean coordinate (src/coordinateset.cpp:214-229)."""
+        c = self.coords
+        if isinstance(c, torch.Tensor):
+            c = c.detach().cpu().numpy()
+        c = np.asarray(c, dtype=np.float64)
+        if c.shape[0] == 0:
+            return float3()
+        m = c.mean(axis=0)
+        return float3(*m)
+
+
+# --------------------------------------------------------------------------- #
+# GridMaker
+# --------------------------------------------------------------------------- #
+class GridMaker(object):
+    """Atoms -> density grid and grid gradient -> atom gradients.
+
+    Same constructor arguments and defaults as the reference's Python class
+    (python/bindings.in.cpp:816-817).
+    """
+
+    def __init__(self, resolution=0.5, dimension=23.5, binary=False, radius_type_indexed=False,
+                 radius_scale=1.0, gaussian_radius_multiple=1.0):
+        self._radius_scale = float(radius_scale)
+        self._grm_arg = float(gaussian_radius_multiple)
+        self._p = _capi.mg_gridmaker()
+        self._init(resolution, dimension, binary, radius_type_indexed)
+
+    def _init(self, resolution, dimension, binary, rti):
+        _capi.check(_lib.mg_gridmaker_init(self._p, resolution, dimension, int(bool(binary)),
+                                           int(bool(rti)), self._radius_scale, self._grm_arg),
+                    "GridMaker")
+
+    # -- accessors (grid_maker.h:88-116) ------------------------------------
+    def get_resolution(self):
+        return float(self._p.resolution)
+
+    def set_resolution(self, res):
+        self._init(res, self._p.dimension, self._p.binary, self._p.radii_type_indexed)
+
+    def get_dimension(self):
+        return float(self._p.dimension)
+
+    def set_dimension(self, d):
+        self._init(self._p.resolution, d, self._p.binary, self._p.radii_type_indexed)
+
+    def get_binary(self):
+        return bool(self._p.binary)
+
+    def set_binary(self, b):
+        self._p.binary = int(bool(b))
+
+    def get_radii_type_indexed(self):
+        return bool(self._p.radii_type_indexed)
+
+    def set_radii_type_indexed(self, b):
+        self._p.radii_type_indexed = int(bool(b))
+
+    def get_radiusmultiple(self):
+        return float(_f32(self._p.radius_scale) * _f32(self._p.final_radius_multiple))
+
+    def get_first_dim(self):
+        return int(self._p.dim)
+
+    def spatial_grid_dimensions(self):
+        d = int(self._p.dim)
+        return (d, d, d)
+
+    def grid_dimensions(self, ntypes):
+        d = int(self._p.dim)
+        return (int(ntypes), d, d, d)
+
+    def get_grid_origin(self, center):
+        c = _to_float3(center)
+        half = _f32(float(self._p.dimension) / 2.0)
+        return float3(_f32(c.x) - half, _f32(c.y) - half, _f32(c.z) - half)
+
+    # -- argument checks ----------------------------------------------------
+    def _check_grid(self, shape, what="Output"):
+        dim = int(self._p.dim)
+        for ax in (1, 2, 3):
+            if shape[ax] != dim:
+                raise IndexError("%s grid dimension incorrect: %d vs %d" % (what, dim, shape[ax]))
+
+    def _check_index_args(self, n, types, radii, out_shape):
+        # src/grid_maker.cpp:39-54
+        self._check_grid(out_shape)
+        if types.shape[0] != n:
+            raise IndexError("type_index does not match number of atoms: %d vs %d"
+                             % (types.shape[0], n))
+        if radii.shape[0] != n:
+            raise IndexError("radii does not match number of atoms: %d vs %d"
+                             % (radii.shape[0], n))
+
+    def _check_vector_args(self, n, types, radii, out_shape):
+        # src/grid_maker.cpp:66-89
+        self._check_grid(out_shape)
+        T = types.shape[1]
+        if types.shape[0] != n:
+            raise IndexError("type_vector does not match number of atoms: %d vs %d"
+                             % (types.shape[0], n))
+        if T != out_shape[0]:
+            raise IndexError("number of types in type_vector does not match number of output "
+                             "channels: %d vs %d" % (T, out_shape[0]))
+        want = T if self._p.radii_type_indexed else n
+        if radii.shape[0] != want:
+            raise IndexError("radii does not match number of %s: %d vs %d"
+                             % ("types" if self._p.radii_type_indexed else "atoms",
+                                radii.shape[0], want))
+
+    @staticmethod
+    def _check_host_types(types_user, ntypes):
+        """The CPU overload throws for an index >= ntypes (src/grid_maker.cpp:172); the
+        check is made for host arrays, where it costs no device synchronisation."""
+        if _is_host(types_user):
+            t = np.asarray(types_user.detach().numpy() if isinstance(types_user, torch.Tensor)
+                           else types_user)
+            if t.size and np.floor(t).max() >= ntypes:
+                raise IndexError("Type index %d larger than allowed %d"
+                                 % (int(np.floor(t).max()), ntypes))
+
+    # -- forward ------------------------------------------------------------
+    def forward(self, *args, **kw):
+        """forward(center, coordinate_set, grid)
+        forward(center, coords, types, radii, grid)          one example
+        forward(centers, coords, types, radii, grid)         padded batch (B leading)
+        ``types`` is 1-D per example for index types, 2-D for type vectors."""
+        if kw:
+            raise TypeError("forward takes positional arguments only")
+        if len(args) == 3:
+            center, cs, grid = args
+            if not isinstance(cs, CoordinateSet):
+                raise TypeError("forward(center, CoordinateSet, grid) expected")
+            types = cs.type_vector if cs.has_vector_types() and cs.size() > 0 else cs.type_index
+            if types is None:
+                types = cs.type_vector
+            return self.forward(center, cs.coords, types, cs.radii, grid)
+        if len(args) != 5:
+            raise TypeError("forward expects 3 or 5 arguments")
+        center, coords, types, radii, grid = args
+        if len(tuple(coords.shape)) == 3:
+            return self._forward_padded(center, coords, types, radii, grid)
+        c = _to_float3(center)
+        a_coords = _Arg(coords, "coords", 2)
+        tdim = len(tuple(types.shape))
+        a_types = _Arg(types, "types", tdim)
+        a_radii = _Arg(radii, "radii", 1)
+        a_out = _Arg(grid, "grid", 4, out=True)
+        n = a_coords.shape[0]
+        if tdim == 1:
+            self._check_index_args(n, a_types, a_radii, a_out.shape)
+            if self._p.radii_type_indexed:
+                raise ValueError("Type indexed radii not supported with index types.")
+            self._check_host_types(types, a_out.shape[0])
+            fn = _lib.mg_forward_index
+        else:
+            self._check_vector_args(n, a_types, a_radii, a_out.shape)
+            fn = _lib.mg_forward_vector
+        code = fn(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr, a_types.ptr, a_radii.ptr,
+                  a_out.shape[0], a_out.ptr, _stream())
+        _capi.check(code, "GridMaker.forward")
+        a_out.finish()
+
+    def _forward_padded(self, centers, coords, types, radii, grid):
+        # include/libmolgrid/grid_maker.h:265-301
+        a_centers = _Arg(centers, "centers", 2)
+        a_coords = _Arg(coords, "coords", 3)
+        tdim = len(tuple(types.shape))
+        if tdim not in (2, 3):
+            raise ValueError("Unsupported types dimension")
+        a_types = _Arg(types, "types", tdim)
+        a_radii = _Arg(radii, "radii", 2)
+        a_out = _Arg(grid, "grid", 5, out=True)
+        B = a_centers.shape[0]
+        for a in (a_coords, a_types, a_radii, a_out):
+            if a.shape[0] != B:
+                raise ValueError("Mismatched batch sizes: %d vs %d" % (a.shape[0], B))
+        n = a_coords.shape[1]
+        if tdim == 2:
+            self._check_index_args(n, _Shape(a_types.shape[1:]), _Shape(a_radii.shape[1:]),
+                                   a_out.shape[1:])
+            if self._p.radii_type_indexed:
+                raise ValueError("Type indexed radii not supported with index types.")
+            self._check_host_types(types, a_out.shape[1])
+            fn = _lib.mg_forward_index
+        else:
+            self._check_vector_args(n, _Shape(a_types.shape[1:]), _Shape(a_radii.shape[1:]),
+                                    a_out.shape[1:])
+            fn = _lib.mg_forward_vector
+        code = fn(self._p, B, None, n, a_centers.ptr, _capi.f3(_Z3), a_coords.ptr, a_types.ptr,
+                  a_radii.ptr, a_out.shape[1], a_out.ptr, _stream())
+        _capi.check(code, "GridMaker.forward")
+        a_out.finish()
+
+    def forward_batch(self, offsets, centers, coords, types, radii, grid):
+        """Ragged batch in one launch: example b owns atoms offsets[b]:offsets[b+1] of the
+        packed arrays; centers (B,3); grid (B,T,D,D,D).  With type-indexed radii,
+        ``radii`` is (B,T)."""
+        off, B, largest, total = _offsets_arg(offsets)
+        cen = _small_device(centers, 3)
+        a_coords = _Arg(coords, "coords", 2)
+        tdim = len(tuple(types.shape))
+        a_types = _Arg(types, "types", tdim)
+        rti = bool(self._p.radii_type_indexed)
+        a_radii = _Arg(radii, "radii", 2 if rti else 1)
+        a_out = _Arg(grid, "grid", 5, out=True)
+        if cen.shape[0] != B or a_out.shape[0] != B:
+            raise ValueError("Mismatched batch sizes: %d vs %d" % (a_out.shape[0], B))
+        if a_coords.shape[0] < total or a_types.shape[0] < total:
+            raise IndexError("atom arrays are shorter than offsets[-1]")
+        self._check_grid(a_out.shape[1:])
+        T = a_out.shape[1]
+        if tdim == 1:
+            if rti:
+                raise ValueError("Type indexed radii not supported with index types.")
+            if a_radii.shape[0] < total:
+                raise IndexError("radii does not match number of atoms")
+            self._check_host_types(types, T)
+            fn = _lib.mg_forward_index
+        else:
+            if a_types.shape[1] != T:
+                raise IndexError("number of types in type_vector does not match number of "
+                                 "output channels: %d vs %d" % (a_types.shape[1], T))
+            if rti and a_radii.shape != (B, T):
+                raise IndexError("radii does not match number of types")
+            if not rti and a_radii.shape[0] < total:
+                raise IndexError("radii does not match number of atoms")
+            fn = _lib.mg_forward_vector
+        code = fn(self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3), a_coords.ptr,
+                  a_types.ptr, a_radii.ptr, T, a_out.ptr, _stream())
+        _capi.check(code, "GridMaker.forward_batch")
+        a_out.finish()
+
+    # -- backward -----------------------------------------------------------
+    def backward(self, *args):
+        """backward(center, coordinate_set, diff, atom_gradients[, type_gradients])
+        backward(center, coords, type_index, radii, diff, atom_gradients)
+        backward(center, coords, type_vectors, radii, diff, atom_gradients, type_gradients)"""
+        if len(args) in (4, 5) and isinstance(args[1], CoordinateSet):
+            center, cs, diff = args[:3]
+            if len(args) == 5:
+                if not cs.has_vector_types():
+                    raise ValueError("Vector types missing from coordinate set")
+                return self.backward(center, cs.coords, cs.type_vector, cs.radii, diff, args[3],
+                                     args[4])
+            if not cs.has_indexed_types():
+                raise ValueError("Index types missing from coordinate set")
+            return self.backward(center, cs.coords, cs.type_index, cs.radii, diff, args[3])
+        if len(args) not in (6, 7):
+            raise TypeError("backward expects 4 to 7 arguments")
+        center, coords, types, radii, diff, agrad = args[:6]
+        c = _to_float3(center)
+        a_coords = _Arg(coords, "coords", 2)
+        tdim = len(tuple(types.shape))
+        a_types = _Arg(types, "types", tdim)
+        a_radii = _Arg(radii, "radii", 1)
+        a_diff = _Arg(diff, "diff", 4)
+        a_ag = _Arg(agrad, "atom_gradients", 2, out=True)
+        n = a_coords.shape[0]
+        dim = int(self._p.dim)
+        if tdim == 1:
+            if len(args) != 6:
+                raise TypeError("index types take no type_gradients argument")
+            # src/grid_maker.cpp:442-452
+            if self._p.radii_type_indexed:
+                raise ValueError("Type indexed radii not supported with index types.")
+            if n != a_types.shape[0]:
+                raise ValueError("Type dimension doesn't equal number of coordinates.")
+            if n != a_ag.shape[0]:
+                raise ValueError("Gradient dimension doesn't equal number of coordinates")
+            if n != a_radii.shape[0]:
+                raise ValueError("Radii dimension doesn't equal number of coordinates")
+            if a_coords.shape[1] != 3 or a_ag.shape[1] != 3:
+                raise ValueError("Need x,y,z,r for coord_radius")
+            for ax in (1, 2, 3):
+                if a_diff.shape[ax] != dim:
+                    raise ValueError("diff does not have correct dimension %d: %d vs %d"
+                                     % (ax, a_diff.shape[ax], dim))
+            if _is_host(types):
+                t = np.asarray(a_types.host.numpy())
+                if t.size and np.round(t).max() >= a_diff.shape[0]:
+                    raise ValueError("Incorrect channel size for diff: %d vs %d"
+                                     % (int(np.round(t).max()), a_diff.shape[0]))
+            code = _lib.mg_backward_index(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr,
+                                          a_types.ptr, a_radii.ptr, a_diff.shape[0], a_diff.ptr,
+                                          a_ag.ptr, _stream())
+            _capi.check(code, "GridMaker.backward")
+            a_ag.finish()
+            return
+        if len(args) != 7:
+            raise TypeError("vector types need a type_gradients argument")
+        a_tg = _Arg(args[6], "type_gradients", 2, out=True)
+        T = a_types.shape[1]
+        # src/grid_maker.cpp:487-498
+        if n != a_types.shape[0]:
+            raise ValueError("Type dimension doesn't equal number of coordinates.")
+        if T != a_diff.shape[0]:
+            raise ValueError("Channels in diff doesn't equal number of types")
+        if n != a_ag.shape[0]:
+            raise ValueError("Atom gradient dimension doesn't equal number of coordinates")
+        if n != a_tg.shape[0]:
+            raise ValueError("Type gradient dimension doesn't equal number of coordinates")
+        if a_tg.shape[1] != T:
+            raise ValueError("Type gradient dimension has wrong number of types")
+        if a_coords.shape[1] != 3 or a_ag.shape[1] != 3:
+            raise ValueError("Need x,y,z,r for coord_radius")
+        if self._p.radii_type_indexed:
+            if T != a_radii.shape[0]:
+                raise ValueError("Radii dimension doesn't equal number of types")
+        elif n != a_radii.shape[0]:
+            raise ValueError("Radii dimension doesn't equal number of coordinates")
+        for ax in (1, 2, 3):
+            if a_diff.shape[ax] != dim:
+                raise ValueError("diff does not have correct dimension %d: %d vs %d"
+                                 % (ax, a_diff.shape[ax], dim))
+        code = _lib.mg_backward_vector(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr,
+                                       a_types.ptr, a_radii.ptr, T, a_diff.ptr, a_ag.ptr,
+                                       a_tg.ptr, _stream())
+        _capi.check(code, "GridMaker.backward")
+        a_ag.finish()
+        a_tg.finish()
+
+    def backward_batch(self, offsets, centers, coords, types, radii, diff, atom_gradients,
+                       type_gradients=None):
+        """Ragged batch in one launch; diff is (B,T,D,D,D); gradients are packed like the
+        atom arrays."""
+        off, B, largest, total = _offsets_arg(offsets)
+        cen = _small_device(centers, 3)
+        a_coords = _Arg(coords, "coords", 2)
+        tdim = len(tuple(types.shape))
+        a_types = _Arg(types, "types", tdim)
+        rti = bool(self._p.radii_type_indexed)
+        a_radii = _Arg(radii, "radii", 2 if rti else 1)
+        a_diff = _Arg(diff, "diff", 5)
+        a_ag = _Arg(atom_gradients, "atom_gradients", 2, out=True)
+        if cen.shape[0] != B or a_diff.shape[0] != B:
+            raise ValueError("Mismatched batch sizes: %d vs %d" % (a_diff.shape[0], B))
+        if a_ag.shape != a_coords.shape or a_coords.shape[1] != 3:
+            raise ValueError("Gradient dimension doesn't equal number of coordinates")
+        if a_coords.shape[0] < total or a_types.shape[0] < total:
+            raise ValueError("atom arrays are shorter than offsets[-1]")
+        dim = int(self._p.dim)
+        for ax in (2, 3, 4):
+            if a_diff.shape[ax] != dim:
+                raise ValueError("diff does not have correct dimension %d: %d vs %d"
+                                 % (ax - 1, a_diff.shape[ax], dim))
+        T = a_diff.shape[1]
+        if tdim == 1:
+            if rti:
+                raise ValueError("Type indexed radii not supported with index types.")
+            code = _lib.mg_backward_index(self._p, B, _ptr(off), largest, _ptr(cen),
+                                          _capi.f3(_Z3), a_coords.ptr, a_types.ptr, a_radii.ptr,
+                                          T, a_diff.ptr, a_ag.ptr, _stream())
+            _capi.check(code, "GridMaker.backward_batch")
+            a_ag.finish()
+            return
+        if type_gradients is None:
+            raise TypeError("vector types need a type_gradients argument")
+        a_tg = _Arg(type_gradients, "type_gradients", 2, out=True)
+        if a_types.shape[1] != T or a_tg.shape != a_types.shape:
+            raise ValueError("Type gradient dimension has wrong number of types")
+        if rti and a_radii.shape != (B, T):
+            raise ValueError("Radii dimension doesn't equal number of types")
+        code = _lib.mg_backward_vector(self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3),
+                                       a_coords.ptr, a_types.ptr, a_radii.ptr, T, a_diff.ptr,
+                                       a_ag.ptr, a_tg.ptr, _stream())
+        _capi.check(code, "GridMaker.backward_batch")
+        a_ag.finish()
+        a_tg.finish()
+
+
+class _Shape(object):
+    """Carries only a ``shape`` for the shared argument checks."""
+
+    def __init__(self, shape):
+        self.shape = tuple(shape)
+
+
+# --------------------------------------------------------------------------- #
+# GridInterpolater
+# --------------------------------------------------------------------------- #
+class GridInterpolater(object):
+    """Trilinear resampling of a 4-D grid through the inverse of a Transform
+    (python/bindings.in.cpp:920-943, include/libmolgrid/grid_interpolater.h)."""
+
+    def __init__(self, in_resolution=0.5, in_dimension=23.5, out_resolution=0.5,
+                 out_dimension=23.5):
+        self.in_resolution = float(in_resolution)
+        self.in_dimension = float(in_dimension)
+        self.out_resolution = float(out_resolution)
+        self.out_dimension = float(out_dimension)
+
+    @staticmethod
+    def _points(dimension, resolution):
+        return int(np.round(_f32(dimension) / _f32(resolution)) + 1)
+
+    @property
+    def in_dim(self):
+        return self._points(self.in_dimension, self.in_resolution)
+
+    @property
+    def out_dim(self):
+        return self._points(self.out_dimension, self.out_resolution)
+
+    def get_in_resolution(self):
+        return self.in_resolution
+
+    def get_out_resolution(self):
+        return self.out_resolution
+
+    def get_in_dimension(self):
+        return self.in_dimension
+
+    def get_out_dimension(self):
+        return self.out_dimension
+
+    def set_in_resolution(self, r):
+        self.in_resolution = float(r)
+
+    def set_out_resolution(self, r):
+        self.out_resolution = float(r)
+
+    def set_in_dimension(self, d):
+        self.in_dimension = float(d)
+
+    def set_out_dimension(self, d):
+        self.out_dimension = float(d)
+
+    def _check(self, in_shape, out_shape, same):
+        # src/grid_interpolater.cpp:55-76
+        if same:
+            raise ValueError("Input and output grid can not be the same in GridInterpolator.")
+        if in_shape[0] != out_shape[0]:
+            raise ValueError("Different channel dimensions for input and output  grids.")
+        if tuple(in_shape[1:]) != (self.in_dim,) * 3:
+            raise ValueError("Input grid wrong dimension. Should be %d along all axes but is "
+                             "%d,%d,%d" % ((self.in_dim,) + tuple(in_shape[1:])))
+        if tuple(out_shape[1:]) != (self.out_dim,) * 3:
+            raise ValueError("Output grid wrong dimension. Should be %d along all axes but is "
+                             "%d,%d,%d" % ((self.out_dim,) + tuple(out_shape[1:])))
+
+    def forward(self, *args, **kw):
+        """forward(in, transform, out)
+        forward(in_center, in, transform, out_center, out)
+        forward(in, out, random_translation=0, random_rotation=False)"""
+        if len(args) == 5:
+            in_center, src, transform, out_center, dst = args
+        elif len(args) >= 2 and not isinstance(args[1], Transform):
+            src, dst = args[:2]
+            rt = args[2] if len(args) > 2 else kw.get("random_translation", 0.0)
+            rr = args[3] if len(args) > 3 else kw.get("random_rotation", False)
+            transform = Transform(_Z3, rt, rr)
+            in_center = out_center = transform.get_rotation_center()
+        elif len(args) == 3:
+            src, transform, dst = args
+            in_center = out_center = transform.get_rotation_center()
+        else:
+            raise TypeError("unsupported GridInterpolater.forward arguments")
+        a_in = _Arg(src, "in", 4)
+        a_out = _Arg(dst, "out", 4, out=True)
+        same = (src is dst) or _same_memory(src, dst)
+        self._check(a_in.shape, a_out.shape, same)
+        code = _lib.mg_interpolate(
+            self.in_resolution, self.in_dimension, self.out_resolution, self.out_dimension, 1,
+            a_in.shape[0], None, _capi.f3(_to_float3(in_center)), a_in.ptr, None,
+            _capi.f4(transform.get_quaternion().as_tuple()), None,
+            _capi.f3(transform.get_rotation_center()), None,
+            _capi.f3(transform.get_translation()), None, _capi.f3(_to_float3(out_center)),
+            a_out.ptr, _stream())
+        _capi.check(code, "GridInterpolater.forward")
+        a_out.finish()
+
+    def forward_batch(self, src, quats, rot_centers, translations, dst, in_centers=None,
+                      out_centers=None):
+        """One launch for a batch: src (B,K,Din,Din,Din) -> dst (B,K,Dout,Dout,Dout) with one
+        transform per example.  Grid centres default to the rotation centres."""
+        a_in = _Arg(src, "in", 5)
+        a_out = _Arg(dst, "out", 5, out=True)
+        B = a_in.shape[0]
+        if a_out.shape[0] != B:
+            raise ValueError("Mismatched batch sizes: %d vs %d" % (a_out.shape[0], B))
+        same = (src is dst) or _same_memory(src, dst)
+        self._check(a_in.shape[1:], a_out.shape[1:], same)
+        q, c, t = (_small_device(quats, 4), _small_device(rot_centers, 3),
+                   _small_device(translations, 3))
+        ic = _small_device(in_centers, 3) if in_centers is not None else c
+        oc = _small_device(out_centers, 3) if out_centers is not None else c
+        for v in (q, c, t, ic, oc):
+            if v.shape[0] != B:
+                raise ValueError("Mismatched batch sizes: %d vs %d" % (v.shape[0], B))
+        code = _lib.mg_interpolate(
+            self.in_resolution, self.in_dimension, self.out_resolution, self.out_dimension, B,
+            a_in.shape[1], _ptr(ic), _capi.f3(_Z3), a_in.ptr, _ptr(q), _capi.f4(_IDQ), _ptr(c),
+            _capi.f3(_Z3), _ptr(t), _capi.f3(_Z3), _ptr(oc), _capi.f3(_Z3), a_out.ptr, _stream())
+        _capi.check(code, "GridInterpolater.forward_batch")
+        a_out.finish()

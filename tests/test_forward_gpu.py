@@ -1,0 +1,190 @@
+"""GPU parity of GridMaker.forward (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import synth
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mg():
+    import libmolgrid_amd
+    return libmolgrid_amd
+
+
+def gpu_forward(mg, gm_args, center, coords, types, radii, ntypes):
+    gm = mg.GridMaker(*gm_args)
+    out = torch.full(gm.grid_dimensions(ntypes), 7.0, device="cuda")  # must be overwritten
+    gm.forward(center, dev(coords), dev(types), dev(radii), out)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def test_density_profile_closed_form(mg):
+    """Same constants as the reference's test_radius_multiples (test/test_gridmaker.py:131-184)."""
+    c = np.zeros((1, 3), np.float32)
+    t = np.zeros(1, np.float32)
+    r = np.ones(1, np.float32)
+    g = gpu_forward(mg, (0.1, 6.0), (0, 0, 0), c, t, r, 1)
+    assert g[0, 30, 30, 30] == pytest.approx(1.0)
+    line = g[0, 30, 30, :]
+    x = np.abs(np.arange(-3, 3.1, .1))
+    gauss = np.exp(-2 * x ** 2)
+    for i in range(20, 41):
+        assert line[i] == pytest.approx(gauss[i], abs=1e-6)
+    for i in list(range(0, 15)) + list(range(45, 61)):
+        assert line[i] == pytest.approx(0, abs=1e-7)
+    quad = 4 * np.exp(-2) * x ** 2 - 12 * np.exp(-2) * x + 9 * np.exp(-2)
+    for i in list(range(15, 20)) + list(range(41, 45)):
+        assert line[i] == pytest.approx(quad[i], abs=1e-5)
+    # radius_scale 0.5, gaussian_radius_multiple 3: Gaussian all the way
+    g = gpu_forward(mg, (0.1, 6.0, False, False, 0.5, 3.0), (0, 0, 0), c, t, r, 1)
+    line = g[0, 30, :, 30]
+    gauss = np.exp(-2 * (x * 2.0) ** 2)
+    for i in range(0, 61):
+        assert line[i] == pytest.approx(gauss[i], abs=1e-5)
+
+
+@pytest.mark.parametrize("res,dimension,ntypes,natoms", [
+    (0.5, 6.0, 3, 20),      # dim 13: partial tiles on every axis
+    (0.5, 12.0, 5, 60),     # dim 25
+    (0.25, 5.75, 2, 15),    # dim 24
+    (1.0, 15.0, 40, 200),   # dim 16, more channels than one LDS pass holds
+    (0.5, 23.5, 28, 300),   # dim 48
+])
+@pytest.mark.parametrize("binary", [False, True])
+def test_small_random_vs_oracle(mg, res, dimension, ntypes, natoms, binary):
+    rng = np.random.default_rng(11 + natoms)
+    coords, types, radii = synth.small_index_case(rng, natoms, ntypes, dimension / 2 + 2.0)
+    types = types + rng.uniform(0, 0.9, natoms).astype(np.float32) * (types >= 0)  # floor()
+    center = rng.uniform(-1, 1, 3).astype(np.float32)
+    ref = oracle.GridMaker(res, dimension, binary).forward(center, coords, types, radii, ntypes)
+    got = gpu_forward(mg, (res, dimension, binary), center, coords, types, radii, ntypes)
+    if binary:
+        assert np.array_equal(got, ref)
+    else:
+        assert_close(got, ref, what="forward")
+
+
+@pytest.mark.parametrize("gm_args", [
+    (0.5, 11.5, False, False, 1.0, -1.5),   # truncated Gaussian, no quadratic tail
+    (0.5, 11.5, True, False, 1.0, -0.5),    # binary sphere wider than its index box
+    (0.5, 11.5, False, False, 1.3, 0.7),    # radius scale + early quadratic
+    (0.5, 11.5, True, False, 0.6, 2.0),
+])
+def test_unusual_radius_multiples(mg, gm_args):
+    rng = np.random.default_rng(5)
+    coords, types, radii = synth.small_index_case(rng, 80, 4, 7.0)
+    ref = oracle.GridMaker(*gm_args).forward((0, 0, 0), coords, types, radii, 4)
+    got = gpu_forward(mg, gm_args, (0, 0, 0), coords, types, radii, 4)
+    if gm_args[2]:
+        assert np.array_equal(got, ref)
+    else:
+        assert_close(got, ref, what="forward")
+
+
+def test_many_atoms_on_one_spot(mg):
+    """More candidates than one LDS list holds: 3000 atoms inside one tile."""
+    rng = np.random.default_rng(3)
+    n = 3000
+    coords = rng.normal(0, 0.3, (n, 3)).astype(np.float32)
+    types = rng.integers(0, 2, n).astype(np.float32)
+    radii = rng.uniform(1.0, 1.5, n).astype(np.float32)
+    ref = oracle.GridMaker(0.5, 7.5).forward((0, 0, 0), coords, types, radii, 2)
+    got = gpu_forward(mg, (0.5, 7.5), (0, 0, 0), coords, types, radii, 2)
+    # thousands of terms per voxel: same summation order, so still tight
+    assert_close(got, ref, rtol=2e-5, what="dense forward")
+
+
+def test_empty_and_ignored_atoms(mg):
+    gm = mg.GridMaker(0.5, 7.5)
+    out = torch.full(gm.grid_dimensions(3), 5.0, device="cuda")
+    gm.forward((0, 0, 0), torch.zeros((0, 3), device="cuda"), torch.zeros(0, device="cuda"),
+               torch.zeros(0, device="cuda"), out)
+    assert float(out.abs().max()) == 0.0
+    coords = dev(np.zeros((4, 3), np.float32))
+    types = dev(np.asarray([-1, -1, 3, 7], np.float32))   # negative and >= ntypes: ignored
+    out.fill_(5.0)
+    gm.forward((0, 0, 0), coords, types, dev(np.ones(4, np.float32)), out)
+    assert float(out.abs().max()) == 0.0
+
+
+def test_config0_vs_oracle(mg):
+    c = synth.config0()
+    ref = oracle.GridMaker(0.5, 23.5).forward((0, 0, 0), c["coords"], c["types"], c["radii"], 28)
+    got = gpu_forward(mg, (0.5, 23.5), (0, 0, 0), c["coords"], c["types"], c["radii"], 28)
+    assert_close(got, ref, what="config 0")
+    refb = oracle.GridMaker(0.5, 23.5, True).forward((0, 0, 0), c["coords"], c["types"],
+                                                    c["radii"], 28)
+    gotb = gpu_forward(mg, (0.5, 23.5, True), (0, 0, 0), c["coords"], c["types"], c["radii"], 28)
+    assert np.array_equal(gotb, refb)
+
+
+@pytest.mark.parametrize("binary", [False, True])
+def test_ragged_batch_with_transform_vs_oracle(mg, binary):
+    """Configuration 1 at a batch the oracle finishes in seconds."""
+    c = synth.config1(nbatch=6)
+    B = len(c["offsets"]) - 1
+    moved_ref = oracle.transform_forward_batch(c["offsets"], c["quats"], c["centers"],
+                                               c["translations"], c["coords"])
+    ref = oracle.GridMaker(0.5, 23.5, binary).forward_batch(
+        c["offsets"], c["centers"], moved_ref, c["types"], c["radii"], 28, nthreads=6)
+    gm = mg.GridMaker(0.5, 23.5, binary)
+    coords = dev(c["coords"])
+    moved = torch.empty_like(coords)
+    mg.transform_batch(c["offsets"], c["quats"], c["centers"], c["translations"], coords, moved)
+    out = torch.full((B,) + gm.grid_dimensions(28), 3.0, device="cuda")
+    gm.forward_batch(c["offsets"], c["centers"], moved, dev(c["types"]), dev(c["radii"]), out)
+    torch.cuda.synchronize()
+    assert np.array_equal(moved.cpu().numpy(), moved_ref)   # same float ops, same order
+    got = out.cpu().numpy()
+    if binary:
+        assert np.array_equal(got, ref)
+    else:
+        assert_close(got, ref, what="config 1")
+
+
+def test_padded_batch_matches_single_calls(mg):
+    rng = np.random.default_rng(9)
+    B, N, T = 3, 50, 4
+    coords = rng.uniform(-5, 5, (B, N, 3)).astype(np.float32)
+    types = rng.integers(-1, T, (B, N)).astype(np.float32)
+    radii = rng.uniform(1, 2, (B, N)).astype(np.float32)
+    centers = rng.uniform(-1, 1, (B, 3)).astype(np.float32)
+    gm = mg.GridMaker(0.5, 9.5)
+    out = torch.empty((B,) + gm.grid_dimensions(T), device="cuda")
+    gm.forward(dev(centers), dev(coords), dev(types), dev(radii), out)
+    for b in range(B):
+        one = torch.empty(gm.grid_dimensions(T), device="cuda")
+        gm.forward(tuple(centers[b]), dev(coords[b]), dev(types[b]), dev(radii[b]), one)
+        assert torch.equal(one, out[b])
+        ref = oracle.GridMaker(0.5, 9.5).forward(centers[b], coords[b], types[b], radii[b], T)
+        assert_close(one.cpu().numpy(), ref, what="padded batch")
+
+
+def test_host_arrays_round_trip(mg):
+    """numpy in, numpy out: staged through the device, same kernel."""
+    rng = np.random.default_rng(2)
+    coords, types, radii = synth.small_index_case(rng, 30, 3, 4.0, frac_ignored=0)
+    gm = mg.GridMaker(0.5, 7.5)
+    out = np.empty(gm.grid_dimensions(3), np.float32)
+    gm.forward((0, 0, 0), coords, types, radii, out)
+    ref = oracle.GridMaker(0.5, 7.5).forward((0, 0, 0), coords, types, radii, 3)
+    assert_close(out, ref, what="host arrays")
+    with pytest.raises(IndexError):     # the CPU overload throws for type >= ntypes
+        gm.forward((0, 0, 0), coords, types + 5, radii, out)
+
+
+def test_repeat_runs_are_bit_identical(mg):
+    c = synth.config1(nbatch=2)
+    gm = mg.GridMaker(0.5, 23.5)
+    args = (c["offsets"], c["centers"], dev(c["coords"]), dev(c["types"]), dev(c["radii"]))
+    a = torch.empty((2,) + gm.grid_dimensions(28), device="cuda")
+    b = torch.empty_like(a)
+    gm.forward_batch(*args, a)
+    gm.forward_batch(*args, b)
+    assert torch.equal(a, b)
