@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the gridding hot path on one MI355X.
+
+A step is one pass over one synthetic batch of 50 ragged complexes
+(configuration 1/2 of BASELINE.json): per-example rigid transform of the atoms,
+forward splat into a 50x28x48^3 float32 tensor, atom-gradient backward against a
+N(0,1) upstream gradient and the un-rotation of those gradients.  All inputs are
+resident in HBM before the timed region.  One JSON line is printed.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def event_ms(fn, iters):
+    """Average milliseconds of fn() over iters launches, timed with events on the
+    stream the kernels are launched on (torch's current stream)."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(cfg, ntypes, nsample, threads):
+    """Oracle (CPU restatement of the reference loops) on the first nsample examples."""
+    import oracle
+    off = cfg["offsets"][: nsample + 1]
+    n = int(off[-1])
+    gm = oracle.GridMaker(0.5, 23.5)
+    rng = np.random.default_rng(1)
+    diff = rng.standard_normal((nsample, ntypes, gm.dim, gm.dim, gm.dim), dtype=np.float32)
+    t0 = time.perf_counter()
+    moved = oracle.transform_forward_batch(off, cfg["quats"], cfg["centers"], cfg["translations"],
+                                           cfg["coords"][:n], nthreads=threads)
+    gm.forward_batch(off, cfg["centers"], moved, cfg["types"][:n], cfg["radii"][:n], ntypes,
+                     nthreads=threads)
+    t1 = time.perf_counter()
+    grads = gm.backward_batch(off, cfg["centers"], moved, cfg["types"][:n], cfg["radii"][:n],
+                              diff, nthreads=threads)
+    oracle.transform_backward_batch(off, cfg["quats"], cfg["centers"], cfg["translations"], grads,
+                                    dotranslate=False, nthreads=threads)
+    t2 = time.perf_counter()
+    return dict(total_s=t2 - t0, forward_s=t1 - t0, backward_s=t2 - t1, atoms=n)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=50)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this library runs on one GPU (examples are independent; a larger job "
+              "splits the batch over processes with no exchange) -- use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import libmolgrid_amd as mg
+    import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+
+    B, T = args.batch, 28
+    cfg = synth.config1(nbatch=B)
+    gm = mg.GridMaker(0.5, 23.5)
+    D = gm.get_first_dim()
+    n_atoms = int(cfg["offsets"][-1])
+
+    # everything resident in HBM before timing
+    offsets = mg.AtomBatch(cfg["offsets"])
+    offsets.dev
+    coords = torch.as_tensor(cfg["coords"]).cuda()
+    types = torch.as_tensor(cfg["types"]).cuda()
+    radii = torch.as_tensor(cfg["radii"]).cuda()
+    quats = torch.as_tensor(cfg["quats"]).cuda()
+    centers = torch.as_tensor(cfg["centers"]).cuda()
+    trans = torch.as_tensor(cfg["translations"]).cuda()
+    moved = torch.empty_like(coords)
+    grid = torch.empty((B, T, D, D, D), device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    diff = torch.randn((B, T, D, D, D), device="cuda", generator=gen)
+    grads = torch.empty_like(coords)
+
+    def k_transform():
+        mg.transform_batch(offsets, quats, centers, trans, coords, moved)
+
+    def k_forward():
+        gm.forward_batch(offsets, centers, moved, types, radii, grid)
+
+    def k_backward():
+        gm.backward_batch(offsets, centers, moved, types, radii, diff, grads)
+
+    def k_unrotate():
+        mg.transform_batch(offsets, quats, centers, trans, grads, grads, dotranslate=False,
+                           inverse=True)
+
+    def step():
+        k_transform()
+        k_forward()
+        k_backward()
+        k_unrotate()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # per-kernel durations (events on the launch stream)
+    it = max(args.steps, 10)
+    ms_fwd = event_ms(k_forward, it)
+    ms_bwd = event_ms(k_backward, it)
+    ms_tr = event_ms(k_transform, it)
+
+    grid_bytes = B * T * D ** 3 * 4
+    fwd_bytes = grid_bytes + n_atoms * 20          # grid written once + coords/type/radius read
+    bwd_bytes = grid_bytes + n_atoms * 20 + n_atoms * 12
+    fwd_gbs = fwd_bytes / (ms_fwd * 1e-3) / 1e9
+    bwd_gbs = bwd_bytes / (ms_bwd * 1e-3) / 1e9
+
+    dominant_fwd = ms_fwd >= ms_bwd
+    roofline = {
+        "kernel": "splat_index_kernel (forward)" if dominant_fwd else "backward_index_kernel",
+        "bound": "hbm",
+        "achieved": round(fwd_gbs if dominant_fwd else bwd_gbs, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
+        "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
+    }
+    kernels = {
+        "forward": {"ms": round(ms_fwd, 4), "grids_per_s": round(B / (ms_fwd * 1e-3), 1),
+                    "GBps": round(fwd_gbs, 1), "hbm_frac": round(fwd_gbs / HBM_PEAK_GBS, 4)},
+        "backward": {"ms": round(ms_bwd, 4),
+                     "atom_grads_per_s": round(n_atoms / (ms_bwd * 1e-3), 1),
+                     "GBps": round(bwd_gbs, 1), "hbm_frac": round(bwd_gbs / HBM_PEAK_GBS, 4)},
+        "transform": {"ms": round(ms_tr, 4)},
+    }
+
+    cpu = None
+    if not args.no_cpu:
+        nsample = min(B, 10)
+        r1 = cpu_baseline(cfg, T, nsample, 1)
+        cpu = {
+            "value": round(nsample / r1["total_s"], 2),
+            "unit": "grids/s",
+            "cores": 1,
+            "kind": "port",
+            "sample": "first %d of the %d examples (%d atoms), transform + forward + backward + "
+                      "gradient un-rotation, single thread like the reference's host loop"
+                      % (nsample, B, r1["atoms"]),
+            "forward_grids_per_s": round(nsample / r1["forward_s"], 2),
+            "backward_atom_grads_per_s": round(r1["atoms"] / r1["backward_s"], 1),
+        }
+        try:
+            import oracle
+            nt = min(oracle.max_threads(), 16)
+            if nt > 1:
+                ns = min(B, max(nsample, 2 * nt))
+                rn = cpu_baseline(cfg, T, ns, nt)
+                cpu["all_cores"] = {"value": round(ns / rn["total_s"], 2), "cores": nt,
+                                    "sample": "first %d examples, OpenMP over the batch" % ns}
+        except Exception as e:  # pragma: no cover
+            cpu["all_cores"] = {"error": str(e)}
+
+    out = {
+        "metric": "grids/sec, 28x48^3 fp32 batch 50, fwd + atom-grad bwd; % of HBM roofline",
+        "value": round(B / (ms_per_step * 1e-3), 1),
+        "unit": "grids/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]+[2]: batch %d ragged complexes (%d atoms), random "
+                               "rotation + translation, 28x48^3 grid at 0.5 A, Gaussian density; "
+                               "transform + forward + atom-gradient backward + un-rotation"
+                               % (B, n_atoms),
+                   "batch": B, "atoms": n_atoms, "grid": [T, D, D, D]},
+        "roofline": roofline,
+        "kernels": kernels,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -6,7 +6,7 @@ C ABI of ``include/molgrid_hip.h``; this package is the Python host side that
 mirrors the reference's ``molgrid`` module for that path.
 """
 from ._capi import LIB_PATH, lib as _lib  # noqa: F401  (fails loudly if the .so is missing)
-from .gridding import (CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
+from .gridding import (AtomBatch, CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
                        float3, set_random_seed, transform_batch)
 
 __version__ = "0.1.0"

@@ -249,22 +249,40 @@ def _small_device(values, width):
     return t
 
 
-def _offsets_arg(offsets, nbatch_hint=None):
-    """(device int32 tensor, nbatch, largest example) for a ragged batch."""
-    if isinstance(offsets, torch.Tensor) and offsets.is_cuda:
-        if offsets.dtype != torch.int32 or not offsets.is_contiguous() or offsets.dim() != 1:
-            raise ValueError("atom offsets on the device must be contiguous int32")
-        host = offsets.cpu().numpy()
-        dev = offsets
-    else:
+class AtomBatch(object):
+    """Atom offsets of a ragged batch, kept on the host and on the device.
+
+    Build it once per batch layout and pass it wherever ``offsets`` is taken:
+    the calls then need no host/device copy of the offsets.
+    """
+
+    def __init__(self, offsets):
+        if isinstance(offsets, torch.Tensor):
+            offsets = offsets.detach().cpu().numpy()
         host = np.ascontiguousarray(offsets, dtype=np.int64)
-        dev = torch.as_tensor(host.astype(np.int32)).to(_device())
-    if host.ndim != 1 or host.size < 1:
-        raise ValueError("atom offsets must be a 1-D array of length batch+1")
-    if np.any(np.diff(host) < 0) or host[0] < 0:
-        raise ValueError("atom offsets must be non-decreasing")
-    largest = int(np.max(np.diff(host))) if host.size > 1 else 0
-    return dev, host.size - 1, max(largest, 1), int(host[-1])
+        if host.ndim != 1 or host.size < 1:
+            raise ValueError("atom offsets must be a 1-D array of length batch+1")
+        if host[0] < 0 or np.any(np.diff(host) < 0):
+            raise ValueError("atom offsets must be non-decreasing")
+        if host[-1] >= 2 ** 31:
+            raise ValueError("too many atoms for 32-bit offsets")
+        self.host = host
+        self.nbatch = host.size - 1
+        self.largest = max(int(np.max(np.diff(host))) if host.size > 1 else 0, 1)
+        self.total = int(host[-1])
+        self._dev = None
+
+    @property
+    def dev(self):
+        if self._dev is None:
+            self._dev = torch.as_tensor(self.host.astype(np.int32)).to(_device())
+        return self._dev
+
+
+def _offsets_arg(offsets):
+    """(device int32 tensor, nbatch, largest example, total atoms) for a ragged batch."""
+    b = offsets if isinstance(offsets, AtomBatch) else AtomBatch(offsets)
+    return b.dev, b.nbatch, b.largest, b.total
 
 
 _Z3 = (0.0, 0.0, 0.0)

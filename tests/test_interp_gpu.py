@@ -1,0 +1,80 @@
+"""GPU parity of GridInterpolater.forward (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import synth
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mg():
+    import libmolgrid_amd
+    return libmolgrid_amd
+
+
+def test_identity_and_translation(mg):
+    """test/test_gridinterp.py:15-108: identity is exact, whole-voxel translation shifts."""
+    rng = np.random.default_rng(1)
+    src = rng.random((3, 13, 13, 13), dtype=np.float32)
+    gi = mg.GridInterpolater(0.5, 6.0, 0.5, 6.0)
+    out = torch.empty((3, 13, 13, 13), device="cuda")
+    gi.forward(dev(src), mg.Transform(), out)
+    assert np.array_equal(out.cpu().numpy(), src)
+    T = mg.Transform(mg.Quaternion(), (0, 0, 0), (0.5, 0, 0))     # one voxel along x
+    gi.forward(dev(src), T, out)
+    got = out.cpu().numpy()
+    np.testing.assert_allclose(got[:, 1:], src[:, :-1], atol=1e-5)
+    assert np.all(got[:, 0] == 0)
+
+
+@pytest.mark.parametrize("case", [
+    (0.5, 6.0, 0.5, 6.0), (0.5, 6.0, 0.25, 4.0), (0.25, 5.0, 0.5, 8.0)])
+def test_random_transform_vs_oracle(mg, case):
+    rng = np.random.default_rng(2)
+    ires, idim, ores, odim = case
+    n_in = int(round(idim / ires)) + 1
+    n_out = int(round(odim / ores)) + 1
+    src = rng.standard_normal((4, n_in, n_in, n_in)).astype(np.float32)
+    q = synth.random_quaternions(rng, 1)[0]
+    center = rng.uniform(-1, 1, 3).astype(np.float32)
+    tr = rng.uniform(-1.5, 1.5, 3).astype(np.float32)
+    in_c = rng.uniform(-0.5, 0.5, 3).astype(np.float32)
+    out_c = rng.uniform(-0.5, 0.5, 3).astype(np.float32)
+    ref = oracle.interpolate(ires, idim, ores, odim, in_c, src, q, center, tr, out_c)
+    gi = mg.GridInterpolater(ires, idim, ores, odim)
+    out = torch.full((4, n_out, n_out, n_out), 5.0, device="cuda")
+    gi.forward(tuple(in_c), dev(src), mg.Transform(mg.Quaternion(*q), center, tr), tuple(out_c),
+               out)
+    assert_close(out.cpu().numpy(), ref, what="interpolate")
+
+
+def test_batch_config4_shape_vs_oracle(mg):
+    """Configuration 4 at a batch the oracle finishes in seconds."""
+    rng = np.random.default_rng(4)
+    B, K, D = 3, 28, 48
+    src = rng.standard_normal((B, K, D, D, D)).astype(np.float32) * (rng.random((B, K, D, D, D))
+                                                                     < 0.2)
+    quats = synth.random_quaternions(rng, B)
+    trans = rng.uniform(-1.5, 1.5, (B, 3)).astype(np.float32)
+    zeros = np.zeros((B, 3), np.float32)
+    ref = oracle.interpolate_batch(0.5, 23.5, 0.5, 23.5, zeros, src, quats, zeros, trans, zeros,
+                                   nthreads=3)
+    gi = mg.GridInterpolater(0.5, 23.5, 0.5, 23.5)
+    out = torch.empty((B, K, D, D, D), device="cuda")
+    gi.forward_batch(dev(src), quats, zeros, trans, out)
+    assert_close(out.cpu().numpy(), ref, what="config 4")
+
+
+def test_argument_errors(mg):
+    gi = mg.GridInterpolater(0.5, 6.0, 0.5, 6.0)
+    g = torch.zeros((2, 13, 13, 13), device="cuda")
+    with pytest.raises(ValueError):
+        gi.forward(g, mg.Transform(), g)
+    with pytest.raises(ValueError):
+        gi.forward(g, mg.Transform(), torch.zeros((3, 13, 13, 13), device="cuda"))
+    with pytest.raises(ValueError):
+        gi.forward(g, mg.Transform(), torch.zeros((2, 13, 13, 12), device="cuda"))
