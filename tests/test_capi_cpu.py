@@ -1,0 +1,176 @@
+"""CPU-side checks of the C ABI and of the host logic above it (no kernel is launched)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def mg():
+    import libmolgrid_amd
+    return libmolgrid_amd
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "molgrid_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mg_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(mg):
+    from libmolgrid_amd import _capi
+    names = declared_functions()
+    assert len(names) >= 10
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), "missing export " + n
+    assert set(_capi.EXPORTED_SYMBOLS) == set(names)
+
+
+def test_error_strings(mg):
+    from libmolgrid_amd import _capi
+    assert _capi.error_string(0) == "success"
+    assert "invalid" in _capi.error_string(_capi.MG_ERR_INVALID_ARGUMENT)
+    assert "range" in _capi.error_string(_capi.MG_ERR_OUT_OF_RANGE)
+    with pytest.raises(IndexError):
+        _capi.check(_capi.MG_ERR_OUT_OF_RANGE, "x")
+    with pytest.raises(ValueError):
+        _capi.check(_capi.MG_ERR_INVALID_ARGUMENT, "x")
+    with pytest.raises(RuntimeError):
+        _capi.check(1, "x")
+
+
+@pytest.mark.parametrize("args", [
+    (0.5, 23.5, False, False, 1.0, 1.0), (0.25, 23.75, True, False, 1.0, 1.0),
+    (0.1, 6.0, False, True, 0.5, 3.0), (0.5, 11.5, False, False, 1.3, -1.5),
+    (0.375, 17.0, False, False, 0.9, 0.7)])
+def test_gridmaker_init_matches_oracle_bit_for_bit(mg, args):
+    g = mg.GridMaker(*args)
+    o = oracle.GridMaker(*args)
+    for f in ("resolution", "dimension", "radius_scale", "gaussian_radius_multiple",
+              "final_radius_multiple", "A", "B", "C", "D", "E", "binary", "radii_type_indexed",
+              "dim"):
+        assert getattr(g._p, f) == getattr(o.p, f), f
+    assert g.grid_dimensions(7) == (7, o.dim, o.dim, o.dim)
+    assert g.spatial_grid_dimensions() == (o.dim,) * 3
+
+
+def test_entry_points_reject_bad_arguments_before_launching(mg):
+    from libmolgrid_amd import _capi
+    lib = _capi.lib
+    g = mg.GridMaker(0.5, 7.5, False, True)._p           # type-indexed radii
+    one = ctypes.c_void_p(16)                             # never dereferenced: rejected first
+    z3 = _capi.f3((0, 0, 0))
+    assert lib.mg_forward_index(g, 1, None, 4, None, z3, one, one, one, 3, one, None) == \
+        _capi.MG_ERR_INVALID_ARGUMENT
+    assert lib.mg_backward_index(g, 1, None, 4, None, z3, one, one, one, 3, one, one, None) == \
+        _capi.MG_ERR_INVALID_ARGUMENT
+    ok = mg.GridMaker(0.5, 7.5)._p
+    assert lib.mg_forward_index(ok, -1, None, 4, None, z3, one, one, one, 3, one, None) == \
+        _capi.MG_ERR_INVALID_ARGUMENT
+    assert lib.mg_forward_index(ok, 1, None, 4, None, z3, None, one, one, 3, one, None) == \
+        _capi.MG_ERR_NULL_POINTER
+    assert lib.mg_forward_index(None, 1, None, 4, None, z3, one, one, one, 3, one, None) == \
+        _capi.MG_ERR_NULL_POINTER
+    q = _capi.f4((1, 0, 0, 0))
+    assert lib.mg_interpolate(0.5, 6.0, 0.5, 6.0, 1, 2, None, z3, one, None, q, None, z3, None,
+                              z3, None, z3, one, None) == _capi.MG_ERR_INVALID_ARGUMENT  # in==out
+    assert lib.mg_interpolate(0.0, 6.0, 0.5, 6.0, 1, 2, None, z3, one, None, q, None, z3, None,
+                              z3, None, z3, ctypes.c_void_p(32), None) == \
+        _capi.MG_ERR_INVALID_ARGUMENT
+    # nothing to do is not an error and launches nothing
+    assert lib.mg_forward_index(ok, 0, None, 4, None, z3, one, one, one, 3, one, None) == 0
+    assert lib.mg_transform_forward(1, None, 0, None, q, None, z3, None, z3, 1, None, None,
+                                    None) == 0
+
+
+def test_host_side_shape_checks_raise_like_the_reference(mg):
+    gm = mg.GridMaker(0.5, 7.5)          # dim 16
+    f = lambda *s: np.zeros(s, np.float32)
+    with pytest.raises(IndexError):       # std::out_of_range, src/grid_maker.cpp:46-48
+        gm.forward((0, 0, 0), f(4, 3), f(4), f(4), f(2, 16, 16, 15))
+    with pytest.raises(IndexError):       # :50
+        gm.forward((0, 0, 0), f(4, 3), f(3), f(4), f(2, 16, 16, 16))
+    with pytest.raises(IndexError):       # :51
+        gm.forward((0, 0, 0), f(4, 3), f(4), f(5), f(2, 16, 16, 16))
+    with pytest.raises(IndexError):       # :81-82
+        gm.forward((0, 0, 0), f(4, 3), f(4, 3), f(4), f(2, 16, 16, 16))
+    with pytest.raises(ValueError):       # :160-162
+        mg.GridMaker(0.5, 7.5, False, True).forward((0, 0, 0), f(4, 3), f(4), f(4),
+                                                    f(2, 16, 16, 16))
+    with pytest.raises(IndexError):       # :84-85 radii per type
+        mg.GridMaker(0.5, 7.5, False, True).forward((0, 0, 0), f(4, 3), f(4, 2), f(4),
+                                                    f(2, 16, 16, 16))
+    with pytest.raises(IndexError):       # type index >= ntypes on host arrays, :172
+        gm.forward((0, 0, 0), f(4, 3), f(4) + 2, f(4), f(2, 16, 16, 16))
+    with pytest.raises(ValueError):       # non-contiguous
+        gm.forward((0, 0, 0), f(4, 3), f(4), f(4), f(2, 16, 16, 32)[..., ::2])
+    with pytest.raises(ValueError):       # batched: mismatched batch sizes, grid_maker.h:271-282
+        gm.forward(f(2, 3), f(3, 4, 3), f(2, 4), f(2, 4), f(2, 2, 16, 16, 16))
+    with pytest.raises(ValueError):       # src/grid_maker.cpp:445-451
+        gm.backward((0, 0, 0), f(4, 3), f(4), f(4), f(2, 16, 16, 16), f(3, 3))
+    with pytest.raises(ValueError):
+        gm.backward((0, 0, 0), f(4, 3), f(4, 2), f(4), f(3, 16, 16, 16), f(4, 3), f(4, 2))
+    gi = mg.GridInterpolater(0.5, 6.0, 0.5, 6.0)
+    g = f(2, 13, 13, 13)
+    with pytest.raises(ValueError):       # src/grid_interpolater.cpp:58
+        gi.forward(g, mg.Transform(), g)
+    with pytest.raises(ValueError):
+        gi.forward(g, mg.Transform(), f(3, 13, 13, 13))
+    with pytest.raises(ValueError):       # include/libmolgrid/transform.h:131-146
+        mg.Transform().forward(f(5, 3), f(4, 3))
+
+
+def test_quaternion_matches_oracle_bit_for_bit(mg):
+    rng = np.random.default_rng(0)
+    for _ in range(20):
+        a, b = rng.normal(size=4).astype(np.float32), rng.normal(size=4).astype(np.float32)
+        qa, qb = mg.Quaternion(*a), mg.Quaternion(*b)
+        assert (qa * qb).as_tuple() == tuple(float(v) for v in oracle.quat_mul(a, b))
+        assert qa.inverse().as_tuple() == tuple(float(v) for v in oracle.quat_inverse(a))
+        p = rng.uniform(-5, 5, 3).astype(np.float32)
+        assert tuple(qa.rotate(*p)) == tuple(float(v) for v in oracle.quat_rotate(a, p))
+        c, t = rng.normal(size=3).astype(np.float32), rng.normal(size=3).astype(np.float32)
+        want = oracle.transform_forward(a, c, t, p[None])[0]
+        assert tuple(qa.transform(*p, c, t)) == tuple(float(v) for v in want)
+        quot = (qa / qb) * qb
+        np.testing.assert_allclose(quot.as_tuple(), a, atol=1e-5)
+    assert mg.Quaternion() == mg.Quaternion(1, 0, 0, 0)
+    assert mg.Quaternion(1, 2, 3, 4).conj().as_tuple() == (1, -2, -3, -4)
+    assert mg.Quaternion(1, 2, 3, 4).norm() == 30
+
+
+def test_transform_constructors(mg):
+    t = mg.Transform()
+    assert t.is_identity() and tuple(t.get_rotation_center()) == (0, 0, 0)
+    q = mg.Quaternion(0, 1, 0, 0)
+    t = mg.Transform(q, (1, 2, 3))
+    assert t.get_quaternion() == q and tuple(t.get_translation()) == (0, 0, 0)
+    mg.set_random_seed(1)
+    a = mg.Transform((0, 1, 1), 10.0, True)
+    mg.set_random_seed(1)
+    b = mg.Transform((0, 1, 1), 10.0, True)
+    assert a.get_quaternion() == b.get_quaternion()
+    assert tuple(a.get_translation()) == tuple(b.get_translation())
+    assert abs(a.get_quaternion().norm() - 1) < 1e-5
+    assert all(abs(v) <= 10 for v in a.get_translation())
+    assert not a.is_identity()
+    c = mg.Transform((0, 0, 0), 0.0, False)
+    assert c.is_identity()
+
+
+def test_coordinate_set(mg):
+    c = np.asarray([[0, 0, 0], [2, 4, 6]], np.float32)
+    cs = mg.CoordinateSet(c, np.asarray([0, 1], np.float32), np.ones(2, np.float32), 2)
+    assert cs.has_indexed_types() and not cs.has_vector_types() and cs.num_types() == 2
+    assert tuple(cs.center()) == (1, 2, 3)
+    cv = mg.CoordinateSet(c, np.eye(2, dtype=np.float32), np.ones(2, np.float32))
+    assert cv.has_vector_types() and cv.num_types() == 2 and len(cv) == 2
+    with pytest.raises(ValueError):
+        mg.CoordinateSet(c, np.zeros(3, np.float32), np.ones(2, np.float32), 2)
