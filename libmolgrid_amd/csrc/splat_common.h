@@ -108,26 +108,33 @@ __device__ __forceinline__ int append_candidates(bool pass, int value, int* s_ca
 
 // Index-box clip of the CPU loops (src/grid_maker.cpp:181-189), packed as
 // lo | hi<<16 per axis.
-__device__ __forceinline__ uint3 pack_clip(const GridArg& g, const SplatGeom& s, float ax, float ay,
-                                           float az, float radius) {
+__device__ __forceinline__ uint3 pack_clip(const GridArg& g, float ox, float oy, float oz, float ax,
+                                           float ay, float az, float radius) {
   float densityrad;
   {
 #pragma clang fp contract(off)
     densityrad = radius * g.radius_scale * g.frm;
   }
   int lo[3], hi[3];
-  bounds_1d(s.ox, ax, densityrad, g.resolution, g.dim, lo[0], hi[0]);
-  bounds_1d(s.oy, ay, densityrad, g.resolution, g.dim, lo[1], hi[1]);
-  bounds_1d(s.oz, az, densityrad, g.resolution, g.dim, lo[2], hi[2]);
+  bounds_1d(ox, ax, densityrad, g.resolution, g.dim, lo[0], hi[0]);
+  bounds_1d(oy, ay, densityrad, g.resolution, g.dim, lo[1], hi[1]);
+  bounds_1d(oz, az, densityrad, g.resolution, g.dim, lo[2], hi[2]);
   return make_uint3((unsigned)lo[0] | ((unsigned)hi[0] << 16),
                     (unsigned)lo[1] | ((unsigned)hi[1] << 16),
                     (unsigned)lo[2] | ((unsigned)hi[2] << 16));
 }
+__device__ __forceinline__ uint3 pack_clip(const GridArg& g, const SplatGeom& s, float ax, float ay,
+                                           float az, float radius) {
+  return pack_clip(g, s.ox, s.oy, s.oz, ax, ay, az, radius);
+}
 
+__device__ __forceinline__ bool inside_clip(int xi, int yi, int zi, uint3 cl) {
+  return xi >= (int)(cl.x & 0xffff) && xi < (int)(cl.x >> 16) &&
+         yi >= (int)(cl.y & 0xffff) && yi < (int)(cl.y >> 16) &&
+         zi >= (int)(cl.z & 0xffff) && zi < (int)(cl.z >> 16);
+}
 __device__ __forceinline__ bool inside_clip(const SplatGeom& s, uint3 cl) {
-  return s.vxi >= (int)(cl.x & 0xffff) && s.vxi < (int)(cl.x >> 16) &&
-         s.vyi >= (int)(cl.y & 0xffff) && s.vyi < (int)(cl.y >> 16) &&
-         s.vzi >= (int)(cl.z & 0xffff) && s.vzi < (int)(cl.z >> 16);
+  return inside_clip(s.vxi, s.vyi, s.vzi, cl);
 }
 
 // Density of one atom at one voxel (calc_point, src/grid_maker.cu:95-130).
