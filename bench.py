@@ -39,6 +39,28 @@ def event_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary
+    (FETCH_SIZE + WRITE_SIZE, KiB per dispatch; calibration factor 1.0, stated in that file).
+    None when the summary is missing or does not list the kernel."""
+    path = os.path.join(ROOT, "profiles", "bench_step_config1_kernel_trace.txt")
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None
+    start = [i for i, l in enumerate(lines) if "FETCH_SIZE_KiB" in l and "WRITE_SIZE_KiB" in l]
+    if not start:
+        return None
+    for l in lines[start[0] + 1:]:
+        parts = l.split()
+        if len(parts) >= 3 and l.startswith(kernel):
+            try:
+                return int((float(parts[-2]) + float(parts[-1])) * 1024)
+            except ValueError:
+                return None
+    return None
+
+
 def cpu_baseline(cfg, ntypes, nsample, threads):
     """Oracle (CPU restatement of the reference loops) on the first nsample examples."""
     import oracle
@@ -153,7 +175,8 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": measured_traffic("splat_index_kernel" if dominant_fwd
+                                    else "backward_index_kernel"),
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
     }
