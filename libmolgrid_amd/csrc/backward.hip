@@ -48,9 +48,14 @@ __device__ __forceinline__ float wave_sum(float v) {
 // once per box so that the inner loop needs no division.
 struct BoxWalk {
   int i, j, k;     // current offset inside the box
+  int off;         // linear element offset of the current voxel inside one grid channel
   int di, dj, dk;  // 64 expressed in (nj*nk, nk, 1) digits
   int nj, nk;
-  __device__ __forceinline__ void start(int lane, int nj_, int nk_) {
+  int step;        // offset advance of one stride when no digit wraps
+  int wrap_k, wrap_j;  // offset corrections when k / j wrap
+  // box origin (lo0, lo1, lo2) inside a dim^3 channel
+  __device__ __forceinline__ void start(int lane, int nj_, int nk_, int lo0, int lo1, int lo2,
+                                        int dim) {
     nj = nj_;
     nk = nk_;
     const int plane = nj * nk;
@@ -62,33 +67,51 @@ struct BoxWalk {
     r = kWave - di * plane;
     dj = r / nk;
     dk = r - dj * nk;
+    off = ((lo0 + i) * dim + lo1 + j) * dim + lo2 + k;
+    step = (di * dim + dj) * dim + dk;
+    wrap_k = dim - nk;             // k -= nk, ++j
+    wrap_j = (dim - nj) * dim;     // j -= nj, ++i
   }
   __device__ __forceinline__ void next() {
     k += dk;
-    if (k >= nk) { k -= nk; ++j; }
+    off += step;
+    if (k >= nk) { k -= nk; ++j; off += wrap_k; }
     j += dj;
-    if (j >= nj) { j -= nj; ++i; }
+    if (j >= nj) { j -= nj; ++i; off += wrap_j; }
     i += di;
   }
 };
 
-// d(density)/d(dist) and the scale that turns (voxel - atom) into the
-// gradient term of one voxel: -(1/dist) * agrad_dist * gridval.  Returns 0
-// where the reference skips the voxel (dist == 0 or beyond the cut-off).
-__device__ __forceinline__ float grad_scale(const GridArg& g, float dist2, float inv_ar2,
-                                            float inv_ar, float frm2, float grm2, float gridval) {
-  if (!(dist2 > 0.f)) return 0.f;
-  const float u = dist2 * inv_ar2;
-  if (!(u <= frm2)) return 0.f;
+// Per-atom constants of the gradient scale.
+struct GradConsts {
+  float inv_ar2;   // 1/ar^2
+  float gauss;     // 4/ar^2            (Gaussian part:  scale = gauss * exp(-2u) * gridval)
+  float quad_a;    // -D/ar^2           (quadratic part: scale = (quad_a + quad_b/dist) * gridval)
+  float quad_b;    // -E/ar
+};
+__device__ __forceinline__ GradConsts grad_consts(const GridArg& g, float ar) {
+  GradConsts c;
+  const float inv_ar = 1.0f / ar;
+  c.inv_ar2 = inv_ar * inv_ar;
+  c.gauss = 4.0f * c.inv_ar2;
+  c.quad_a = -g.D * c.inv_ar2;
+  c.quad_b = -g.E * inv_ar;
+  return c;
+}
+
+// Scale that turns (voxel - atom) into the gradient term of one voxel:
+// -(1/dist) * d(density)/d(dist) * gridval (density_grad_dist and accumulate_atom_gradient,
+// src/grid_maker.cu:881-919).  With u = dist^2/ar^2:
+//   Gaussian, u <= grm^2:  d/d(dist) = -4 dist/ar^2 exp(-2u)   ->  4/ar^2 exp(-2u) gridval
+//   quadratic tail:        d/d(dist) = (D dist/ar + E)/ar      -> -(D/ar^2 + E/(ar dist)) gridval
+// and 0 where the reference skips the voxel (dist == 0 or beyond the cut-off).
+__device__ __forceinline__ float grad_scale(const GradConsts& c, float dist2, float frm2,
+                                            float grm2, float gridval) {
+  const float u = dist2 * c.inv_ar2;
+  const float e = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
   const float rinv = __builtin_amdgcn_rsqf(dist2);
-  const float dist = dist2 * rinv;
-  float agd;
-  if (u <= grm2) {
-    agd = -4.0f * dist * inv_ar2 * __builtin_amdgcn_exp2f(u * kNeg2Log2e);
-  } else {
-    agd = (g.D * dist * inv_ar + g.E) * inv_ar;
-  }
-  return -(agd * gridval) * rinv;
+  const float s = (u <= grm2) ? c.gauss * e : fmaf(c.quad_b, rinv, c.quad_a);
+  return (dist2 > 0.f && u <= frm2) ? s * gridval : 0.f;
 }
 
 template <bool BINARY>
@@ -127,25 +150,25 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
         densityrad = radius * g.radius_scale * g.frm;
         ar = radius * g.radius_scale;
       }
-      const float inv_ar = 1.0f / ar;
-      const float inv_ar2 = inv_ar * inv_ar;
+      const GradConsts gc = grad_consts(g, ar);
       int lo0, hi0, lo1, hi1, lo2, hi2;
       bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
       bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
       bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
       const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
       if (ni > 0 && nj > 0 && nk > 0) {
-        const float* chan = diff_b + (size_t)(int)tf * chan_stride;
+        const char* chan = reinterpret_cast<const char*>(diff_b + (size_t)(int)tf * chan_stride);
         BoxWalk w;
-        w.start(lane, nj, nk);
+        w.start(lane, nj, nk, lo0, lo1, lo2, dim);
         for (; w.i < ni; w.next()) {
           const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
           const float dx = grid_coord(ox, xi, g.resolution) - ax;
           const float dy = grid_coord(oy, yi, g.resolution) - ay;
           const float dz = grid_coord(oz, zi, g.resolution) - az;
           const float dist2 = dx * dx + dy * dy + dz * dz;
-          const float gv = chan[((size_t)xi * dim + yi) * dim + zi];
-          const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, gv);
+          // one channel of the grid is < 4 GiB: a 32-bit byte offset from the uniform base
+          const float gv = *reinterpret_cast<const float*>(chan + (unsigned)w.off * 4u);
+          const float sc = grad_scale(gc, dist2, frm2, grm2, gv);
           gx = fmaf(dx, sc, gx);
           gy = fmaf(dy, sc, gy);
           gz = fmaf(dz, sc, gz);
@@ -202,8 +225,8 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         ar = radius * g.radius_scale;
         ar2 = ar * ar;
       }
-      const float inv_ar = 1.0f / ar;
-      const float inv_ar2 = inv_ar * inv_ar;
+      const GradConsts gc = grad_consts(g, ar);
+      const float inv_ar2 = gc.inv_ar2;
       int lo0, hi0, lo1, hi1, lo2, hi2;
       bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
       bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
@@ -217,7 +240,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         for (int t = 0; t < TG; ++t) tg[t] = 0.f;
         if (any) {
           BoxWalk w;
-          w.start(lane, nj, nk);
+          w.start(lane, nj, nk, lo0, lo1, lo2, dim);
           for (; w.i < ni; w.next()) {
             const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
             const float dx = grid_coord(ox, xi, g.resolution) - ax;
@@ -225,7 +248,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
             const float dz = grid_coord(oz, zi, g.resolution) - az;
             const float dist2 = dx * dx + dy * dy + dz * dz;
             const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
-            const float* p = diff_b + (size_t)cbase * chan_stride + ((size_t)xi * dim + yi) * dim + zi;
+            const float* p = diff_b + (size_t)cbase * chan_stride + w.off;
             float weighted = 0.f;  // sum_t weight_t * diff_t at this voxel
 #pragma unroll
             for (int t = 0; t < TG; ++t) {
@@ -235,7 +258,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
                 weighted = fmaf(tv[cbase + t], gv, weighted);
               }
             }
-            const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, weighted);
+            const float sc = grad_scale(gc, dist2, frm2, grm2, weighted);
             gx = fmaf(dx, sc, gx);
             gy = fmaf(dy, sc, gy);
             gz = fmaf(dz, sc, gz);
@@ -261,8 +284,8 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
           ar = radius * g.radius_scale;
           ar2 = ar * ar;
         }
-        const float inv_ar = 1.0f / ar;
-        const float inv_ar2 = inv_ar * inv_ar;
+        const GradConsts gc = grad_consts(g, ar);
+        const float inv_ar2 = gc.inv_ar2;
         int lo0, hi0, lo1, hi1, lo2, hi2;
         bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
         bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
@@ -272,17 +295,17 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         if (ni > 0 && nj > 0 && nk > 0) {
           const float* chan = diff_b + (size_t)t * chan_stride;
           BoxWalk w;
-          w.start(lane, nj, nk);
+          w.start(lane, nj, nk, lo0, lo1, lo2, dim);
           for (; w.i < ni; w.next()) {
             const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
             const float dx = grid_coord(ox, xi, g.resolution) - ax;
             const float dy = grid_coord(oy, yi, g.resolution) - ay;
             const float dz = grid_coord(oz, zi, g.resolution) - az;
             const float dist2 = dx * dx + dy * dy + dz * dz;
-            const float gv = chan[((size_t)xi * dim + yi) * dim + zi];
+            const float gv = chan[w.off];
             const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
             tgt = fmaf(val, gv, tgt);
-            const float sc = grad_scale(g, dist2, inv_ar2, inv_ar, frm2, grm2, gv);
+            const float sc = grad_scale(gc, dist2, frm2, grm2, gv);
             tx = fmaf(dx, sc, tx);
             ty = fmaf(dy, sc, ty);
             tz = fmaf(dz, sc, tz);

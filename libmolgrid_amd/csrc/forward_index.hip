@@ -1,7 +1,8 @@
-// Forward density splat for index-typed atoms on gfx950.
+// Forward density splat on gfx950: index-typed atoms, and vector-typed atoms with per-atom radii.
 //
-// One workgroup of four waves owns a column of the grid: 4 x 4 voxels in (x, y)
-// and up to 48 voxels along z, for every channel.
+// One workgroup of four waves works through three neighbouring columns of the grid, one after the
+// other; a column is 4 x 4 voxels in (x, y) and up to 48 voxels along z, for every channel.  The
+// atom scan (and, in the common case, the record building) is done once for the three columns.
 //   scan    each wave walks a quarter of the example's atoms (loads batched four
 //           deep), keeps those whose density support touches the column's box
 //           and compacts their indices, in ascending order, into its own LDS
@@ -17,7 +18,11 @@
 //           out as full z rows (768 contiguous bytes per channel and x), which is
 //           the pattern the HBM write path sustains best; nothing is memset.
 // Per voxel the contributions are added in ascending atom order, as in the CPU
-// loop (src/grid_maker.cpp:170-211).
+// loops (src/grid_maker.cpp:170-211, 226-270).
+//
+// Vector types (VEC): every atom feeds all channels, so the splat step multiplies the atom's
+// density into all 28 register sums with the atom's weights, which are read through
+// wave-uniform (scalar) loads; binary mode adds the bare weight, in atom order -> bit exact.
 #include "kernels.h"
 #include "splat_common.h"
 
@@ -28,6 +33,7 @@ namespace {
 constexpr int kColXY = 4;                        // column is 4 x 4 voxels in x, y
 constexpr int kBlocksPerWave = 3;                // 4x4x4 blocks per wave
 constexpr int kColWaves = 4;
+constexpr int kColsPerGroup = 3;                // columns (consecutive in y) sharing one atom scan
 constexpr int kColThreads = kColWaves * kWave;   // 256
 constexpr int kSlabZ = kColWaves * kBlocksPerWave * 4;  // 48 voxels of z per workgroup
 constexpr int kRegChannels = 28;                 // channel sums kept in registers per voxel
@@ -38,24 +44,50 @@ constexpr int kSuper = 4096;                     // atoms scanned per pass
 constexpr int kSeg = kSuper / kColWaves;         // per wave
 constexpr int kRecChunk = 256;
 
+// A float that is the same in every lane, moved to a scalar register so that it does not occupy
+// a vector register for the whole kernel.
+__device__ __forceinline__ float uniform(float v) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+
+// The 28 channel sums of one voxel are addressed with a wave-uniform channel index, which the
+// compiler turns into scalar-indexed register moves.  Register tuples come in sizes 16 and 12 (not
+// 28), so each voxel keeps two plain arrays (lo: channels 0-15, hi: 16-27) selected by a scalar
+// branch: 28 registers where one array of 28 would take 32.
+constexpr int kLoChannels = 16;
+constexpr int kHiChannels = kRegChannels - kLoChannels;
+#define MG_SUMS_DECL(name) float name##_lo[kLoChannels], name##_hi[kHiChannels]
+#define MG_SUMS_AT(name, c) ((c) < kLoChannels ? name##_lo[(c) < kLoChannels ? (c) : 0] \
+                                               : name##_hi[(c) < kLoChannels ? 0 : (c) - kLoChannels])
+
+template <bool BINARY>
+__device__ __forceinline__ void sums_add(float (&lo)[kLoChannels], float (&hi)[kHiChannels], int t,
+                                         float val) {
+  if (t < kLoChannels) lo[t] = BINARY ? fmaxf(lo[t], val) : lo[t] + val;
+  else hi[t - kLoChannels] = BINARY ? fmaxf(hi[t - kLoChannels], val) : hi[t - kLoChannels] + val;
+}
+
 // LDS-only barrier: outstanding global stores are not waited for.
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <bool BINARY, bool EXACT>
-__global__ __launch_bounds__(kColThreads) void splat_index_kernel(
+// `types` is type_index [n] (VEC = false) or type_vector [n, ntypes] (VEC = true)
+template <bool BINARY, bool EXACT, bool VEC>
+__global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) void splat_column_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
-    const float* __restrict__ type_index, const float* __restrict__ radii,
+    const float* __restrict__ types, const float* __restrict__ radii,
     float* __restrict__ out, int cols_per_side, int vec_store) {
   __shared__ unsigned short s_idx[kColWaves][kSeg];
   __shared__ int s_wcount[kColWaves];
   __shared__ float4 s_rec[kRecChunk];            // x, y, z, (ar^2 | 1/ar^2)
-  __shared__ unsigned char s_rectype[kRecChunk];
+  __shared__ unsigned char s_rectype[VEC ? 1 : kRecChunk];   // channel of the record (index types)
+  __shared__ int s_recatom[VEC ? kRecChunk : 1];             // atom of the record (vector types)
   __shared__ uint4 s_clip[EXACT ? kRecChunk : 1];  // index box + ar, EXACT only
   __shared__ float4 s_mini[kColWaves][kWave];
   __shared__ uint4 s_miniclip[EXACT ? kColWaves : 1][EXACT ? kWave : 1];
-  __shared__ unsigned char s_minitype[kColWaves][kWave + 4];
+  __shared__ unsigned char s_minitype[VEC ? 1 : kColWaves][VEC ? 1 : kWave + 4];
+  __shared__ int s_miniatom[VEC ? kColWaves : 1][VEC ? kWave + 4 : 1];
   __shared__ __align__(16) float s_stage[2 * kStageCh * kPlane];
 
   const int tid = threadIdx.x;
@@ -65,241 +97,340 @@ __global__ __launch_bounds__(kColThreads) void splat_index_kernel(
   int begin, end;
   example_range(batch, b, begin, end);
   const float3 center = load3(centers, b);
-  const float ox = center.x - g.half_dimension;
-  const float oy = center.y - g.half_dimension;
-  const float oz = center.z - g.half_dimension;
+  const float ox = uniform(center.x - g.half_dimension);
+  const float oy = uniform(center.y - g.half_dimension);
+  const float oz = uniform(center.z - g.half_dimension);
   const int dim = g.dim;
 
-  // which column / z slab this workgroup owns
-  const int ncols = cols_per_side * cols_per_side;
-  const int slab = blockIdx.x / ncols;
-  const int col = blockIdx.x - slab * ncols;
-  const int x0 = (col / cols_per_side) * kColXY, y0 = (col % cols_per_side) * kColXY;
+  // which row of columns / z slab this workgroup owns: kColsPerGroup columns, consecutive in y
+  const int groups_per_row = (cols_per_side + kColsPerGroup - 1) / kColsPerGroup;
+  const int ngroups = cols_per_side * groups_per_row;
+  const int slab = blockIdx.x / ngroups;
+  const int grp = blockIdx.x - slab * ngroups;
+  const int x0 = (grp / groups_per_row) * kColXY;
+  const int gy0 = (grp % groups_per_row) * (kColXY * kColsPerGroup);
   const int z0 = slab * kSlabZ;
   const int zend = min(z0 + kSlabZ, dim);          // exclusive
 
   const int lx = lane >> 4, ly = (lane >> 2) & 3, lz = lane & 3;
-  const int vxi = x0 + lx, vyi = y0 + ly;
-  const bool xy_live = vxi < dim && vyi < dim;
-  const float vx = grid_coord(ox, vxi, g.resolution), vy = grid_coord(oy, vyi, g.resolution);
-  // box of the column (first/last voxel centre inside the grid)
-  const float clx = grid_coord(ox, x0, g.resolution), cly = grid_coord(oy, y0, g.resolution);
-  const float clz = grid_coord(oz, z0, g.resolution);
-  const float chx = grid_coord(ox, min(x0 + kColXY, dim) - 1, g.resolution);
-  const float chy = grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution);
-  const float chz = grid_coord(oz, zend - 1, g.resolution);
+  const int vxi = x0 + lx;
+  const float vx = grid_coord(ox, vxi, g.resolution);
+  // box of the whole group (first/last voxel centre inside the grid)
+  const float clx = uniform(grid_coord(ox, x0, g.resolution));
+  const float clz = uniform(grid_coord(oz, z0, g.resolution));
+  const float chx = uniform(grid_coord(ox, min(x0 + kColXY, dim) - 1, g.resolution));
+  const float chz = uniform(grid_coord(oz, zend - 1, g.resolution));
+  const float gly = uniform(grid_coord(oy, gy0, g.resolution));
+  const float ghy = uniform(grid_coord(oy, min(gy0 + kColXY * kColsPerGroup, dim) - 1, g.resolution));
 
-  const float frm2 = g.frm * g.frm;
-  const float grm2 = g.grm * g.grm;
+  const float frm2 = uniform(g.frm * g.frm);
+  const float grm2 = uniform(g.grm * g.grm);
   const float cull_mult = BINARY ? 1.0f : g.frm;  // support radius / ar
   const size_t chan_stride = (size_t)dim * dim * dim;
   float* out_b = out + (size_t)b * g.ntypes * chan_stride;
 
   const int dump_off = lx * (4 * kRowPad) + ly * kRowPad + wave * kBlocksPerWave * 4 + lz;
 
+  int segstart[kColWaves + 1];
+  int ncand = 0;
+
+  // ---- scan: atoms [s0, s1) against the group's box -> per-wave index segments --------------
+  // Each wave takes a contiguous quarter of the range and keeps up to kSeg survivors (offsets
+  // from s0 as 16-bit values, so s1 - s0 <= 65536).  Returns false if a segment overflowed.
+  auto scan = [&](int s0, int s1) -> bool {
+    const int quarter = (s1 - s0 + kColWaves - 1) / kColWaves;
+    int wcnt = 0;
+    const int wb = s0 + wave * quarter, we = min(s1, wb + quarter);
+    constexpr int U = 2;
+    for (int a0 = wb; a0 < we; a0 += kWave * U) {
+      float rr[U], cx[U], cy[U], cz[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int a = min(a0 + u * kWave + lane, we - 1);
+        rr[u] = radii[a];
+        cx[u] = coords[3 * a];
+        cy[u] = coords[3 * a + 1];
+        cz[u] = coords[3 * a + 2];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int a = a0 + u * kWave + lane;
+        const float reach = rr[u] * g.radius_scale * cull_mult;
+        const bool p = (a < we) && box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy,
+                                                 chz) <= reach * reach * kCullSlack;
+        const unsigned long long m = __ballot(p);
+        const int pos = wcnt + __popcll(m & ((1ull << lane) - 1ull));
+        if (p && pos < kSeg) s_idx[wave][pos] = (unsigned short)(a - s0);
+        wcnt += __popcll(m);
+      }
+    }
+    if (lane == 0) s_wcount[wave] = wcnt;
+    __syncthreads();
+    segstart[0] = 0;
+    bool fits = true;
+#pragma unroll
+    for (int w = 0; w < kColWaves; ++w) {
+      const int c = __builtin_amdgcn_readfirstlane(s_wcount[w]);  // keep in SGPRs
+      fits = fits && c <= kSeg;
+      segstart[w + 1] = segstart[w] + c;
+    }
+    ncand = segstart[kColWaves];
+    lds_barrier();   // every wave has read the counts before any of them scans again
+    return fits;
+  };
+
+  // ---- records: candidates [c0, c0 + m) of the current scan -> 16-byte LDS records -----------
+  auto build_records = [&](int s0, int c0, int m, int cbase, int nchan) {
+    if (tid < m) {
+      const int gi = c0 + tid;
+      int w = 0;
+#pragma unroll
+      for (int k = 1; k < kColWaves; ++k) w += (gi >= segstart[k]) ? 1 : 0;
+      const int a = s0 + s_idx[w][gi - segstart[w]];
+      const float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
+      const float radius = radii[a];
+      const float tf = VEC ? 0.f : floorf(types[a]) - (float)cbase;
+      const bool typed = VEC || (tf >= 0.f && tf < (float)nchan);
+      float ar, ar2;
+      {
+#pragma clang fp contract(off)
+        ar = radius * g.radius_scale;
+        ar2 = ar * ar;
+      }
+      // an atom of another channel group (or an ignored one) can never hit
+      const float w4 = typed ? (BINARY ? ar2 : 1.0f / ar2) : (BINARY ? -1.0f : INFINITY);
+      s_rec[tid] = make_float4(ax, ay, az, w4);
+      if (VEC) s_recatom[tid] = a;
+      else s_rectype[tid] = typed ? (unsigned char)(int)tf : 0;
+      if (EXACT) {
+        const uint3 cl = pack_clip(g, ox, oy, oz, ax, ay, az, radius);
+        s_clip[tid] = make_uint4(cl.x, cl.y, cl.z, __float_as_uint(ar));
+      }
+    }
+    __syncthreads();
+  };
+
+  // Common case: the survivors of the whole example fit the per-wave segments -> one scan shared
+  // by all columns of the group; if they also fit one record chunk and the channels one register
+  // group, the records are shared as well.  Otherwise atoms are taken in passes of kSuper (whose
+  // survivors always fit) and every column scans again.
+  bool one_pass = false;
+  bool records_cached = false;
+  if (end - begin <= 65536) {
+    one_pass = scan(begin, end);
+    if (one_pass && ncand <= kRecChunk && g.ntypes <= kRegChannels) {
+      build_records(begin, 0, ncand, 0, g.ntypes);
+      records_cached = true;
+    }
+  }
+  const int pass_len = one_pass ? max(end - begin, 1) : kSuper;
+
   for (int cbase = 0; cbase < g.ntypes; cbase += kRegChannels) {
     const int nchan = min(kRegChannels, g.ntypes - cbase);
-    float acc0[kRegChannels], acc1[kRegChannels], acc2[kRegChannels];
-#pragma unroll
-    for (int c = 0; c < kRegChannels; ++c) acc0[c] = acc1[c] = acc2[c] = 0.f;
+    const bool full_group = nchan == kRegChannels;
+    for (int col = 0; col < kColsPerGroup; ++col) {
+      const int y0 = gy0 + col * kColXY;
+      if (y0 >= dim) break;
+      const int vyi = y0 + ly;
+      const bool xy_live = vxi < dim && vyi < dim;
+      const float vy = grid_coord(oy, vyi, g.resolution);
+      const float cly = uniform(grid_coord(oy, y0, g.resolution));
+      const float chy = uniform(grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution));
 
-    for (int s0 = begin; s0 < end; s0 += kSuper) {
-      const int send = min(end, s0 + kSuper);
-      // ---- scan --------------------------------------------------------------
-      int wcnt = 0;
-      {
-        const int wb = s0 + wave * kSeg, we = min(send, wb + kSeg);
-        constexpr int U = 2;
-        for (int a0 = wb; a0 < we; a0 += kWave * U) {
-          float rr[U], cx[U], cy[U], cz[U];
+      MG_SUMS_DECL(acc0);
+      MG_SUMS_DECL(acc1);
+      MG_SUMS_DECL(acc2);
 #pragma unroll
-          for (int u = 0; u < U; ++u) {
-            const int a = min(a0 + u * kWave + lane, we - 1);
-            rr[u] = radii[a];
-            cx[u] = coords[3 * a];
-            cy[u] = coords[3 * a + 1];
-            cz[u] = coords[3 * a + 2];
-          }
+      for (int c = 0; c < kLoChannels; ++c) acc0_lo[c] = acc1_lo[c] = acc2_lo[c] = 0.f;
 #pragma unroll
-          for (int u = 0; u < U; ++u) {
-            const int a = a0 + u * kWave + lane;
-            const float reach = rr[u] * g.radius_scale * cull_mult;
-            const bool p = (a < we) && box_distance2(cx[u], cy[u], cz[u], clx, cly, clz, chx, chy,
-                                                     chz) <= reach * reach * kCullSlack;
-            const unsigned long long m = __ballot(p);
-            if (p) s_idx[wave][wcnt + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short)(a - s0);
-            wcnt += __popcll(m);
+      for (int c = 0; c < kHiChannels; ++c) acc0_hi[c] = acc1_hi[c] = acc2_hi[c] = 0.f;
+
+      for (int s0 = begin; s0 < end; s0 += pass_len) {
+        if (!one_pass) scan(s0, min(end, s0 + kSuper));
+        for (int c0 = 0; c0 < ncand; c0 += kRecChunk) {
+          const int m = min(kRecChunk, ncand - c0);
+          if (!records_cached) build_records(s0, c0, m, cbase, nchan);
+
+          // ---- cull per 4x4x4 block, then splat ----------------------------------
+#pragma unroll
+          for (int blk = 0; blk < kBlocksPerWave; ++blk) {
+            const int zb = z0 + (wave * kBlocksPerWave + blk) * 4;
+            if (zb >= zend) continue;
+            const float blz = uniform(grid_coord(oz, zb, g.resolution));
+            const float bhz = uniform(grid_coord(oz, min(zb + 4, zend) - 1, g.resolution));
+            const int vzi = zb + lz;
+            const bool live = xy_live && vzi < zend;
+            const float vz = grid_coord(oz, vzi, g.resolution);
+            for (int r0 = 0; r0 < m; r0 += kWave) {
+              const int i = r0 + lane;
+              bool pass = false;
+              float4 rec = make_float4(0.f, 0.f, 0.f, 0.f);
+              if (i < m) {
+                rec = s_rec[i];
+                const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
+                pass = BINARY ? (d2 <= rec.w * kCullSlack) : (d2 * rec.w <= frm2 * kCullSlack);
+              }
+              const unsigned long long bm = __ballot(pass);
+              const int n = __popcll(bm);
+              if (n == 0) continue;
+              if (pass) {
+                const int p = __popcll(bm & ((1ull << lane) - 1ull));
+                s_mini[wave][p] = rec;
+                if (VEC) s_miniatom[wave][p] = s_recatom[i];
+                else s_minitype[wave][p] = s_rectype[i];
+                if (EXACT) s_miniclip[wave][p] = s_clip[i];
+              }
+              const float4* mp = s_mini[wave];
+              auto tag = [&](int k) -> int { return VEC ? s_miniatom[wave][k] : (int)s_minitype[wave][k]; };
+              auto body = [&](const float4& r, int tt, int it) {
+                const int t = __builtin_amdgcn_readfirstlane(tt);   // channel, or atom (VEC)
+                bool inside = live;
+                float ar = 0.f;
+                if (EXACT) {
+                  const uint4 cl = s_miniclip[wave][it];
+                  inside = inside && inside_clip(vxi, vyi, vzi, make_uint3(cl.x, cl.y, cl.z));
+                  ar = __uint_as_float(cl.w);
+                }
+                float val = density<BINARY, EXACT>(g, vx - r.x, vy - r.y, vz - r.z, r.w, ar, frm2, grm2);
+                if (!inside) val = 0.f;
+                if (VEC) {
+                  const float* __restrict__ tv = types + (size_t)t * g.ntypes + cbase;
+                  // the atom's weights, through wave-uniform loads issued together
+                  float wgt[kRegChannels];
+                  if (full_group && (vec_store & 2)) {   // 16-byte aligned rows: seven 4-wide loads
+                    const float4* __restrict__ tv4 = reinterpret_cast<const float4*>(tv);
+#pragma unroll
+                    for (int q = 0; q < kRegChannels / 4; ++q) {
+                      const float4 w4 = tv4[q];
+                      wgt[4 * q] = w4.x; wgt[4 * q + 1] = w4.y; wgt[4 * q + 2] = w4.z; wgt[4 * q + 3] = w4.w;
+                    }
+                  } else if (full_group) {
+#pragma unroll
+                    for (int c = 0; c < kRegChannels; ++c) wgt[c] = tv[c];
+                  } else {
+#pragma unroll
+                    for (int c = 0; c < kRegChannels; ++c) wgt[c] = c < nchan ? tv[c] : 0.f;
+                  }
+                  auto weigh = [&](float (&lo)[kLoChannels], float (&hi)[kHiChannels]) {
+#pragma unroll
+                    for (int c = 0; c < kRegChannels; ++c) {
+                      float& sum = c < kLoChannels ? lo[c < kLoChannels ? c : 0]
+                                                   : hi[c < kLoChannels ? 0 : c - kLoChannels];
+                      // binary occupancy adds the weight itself where the atom covers the voxel
+                      if (BINARY) sum += (val != 0.f) ? wgt[c] : 0.f;
+                      else sum = fmaf(val, wgt[c], sum);
+                    }
+                  };
+                  if (blk == 0) weigh(acc0_lo, acc0_hi);
+                  else if (blk == 1) weigh(acc1_lo, acc1_hi);
+                  else weigh(acc2_lo, acc2_hi);
+                } else {
+                  // binary occupancy stores 1 where any atom covers the voxel
+                  if (blk == 0) sums_add<BINARY>(acc0_lo, acc0_hi, t, val);
+                  else if (blk == 1) sums_add<BINARY>(acc1_lo, acc1_hi, t, val);
+                  else sums_add<BINARY>(acc2_lo, acc2_hi, t, val);
+                }
+              };
+              // software pipelined: the next record is in flight while this one is evaluated
+              float4 cur = mp[0];
+              int ct = tag(0);
+              int it = 0;
+              for (; it + 2 <= n; it += 2) {
+                const float4 r1 = mp[it + 1];
+                const int t1 = tag(it + 1);
+                body(cur, ct, it);
+                cur = mp[min(it + 2, kWave - 1)];
+                ct = tag(it + 2);
+                body(r1, t1, it + 1);
+              }
+              if (it < n) body(cur, ct, it);
+            }
           }
+          if (!records_cached) lds_barrier();   // records are rebuilt next round
         }
       }
-      if (lane == 0) s_wcount[wave] = wcnt;
-      __syncthreads();
-      int segstart[kColWaves + 1];
-      segstart[0] = 0;
-#pragma unroll
-      for (int w = 0; w < kColWaves; ++w) segstart[w + 1] = segstart[w] + s_wcount[w];
-      const int ncand = segstart[kColWaves];
 
-      for (int c0 = 0; c0 < ncand; c0 += kRecChunk) {
-        // ---- records -----------------------------------------------------------
-        const int m = min(kRecChunk, ncand - c0);
-        if (tid < m) {
-          const int gi = c0 + tid;
-          int w = 0;
+      // ---- store: four channels per round through a double-buffered LDS stage ----
+      // fixed positions of this thread in the staged write-out (float4 granules)
+      constexpr int kItems = kStageCh * 16 * (kSlabZ / 4);               // 768 per round
+      constexpr int kPer = (kItems + kColThreads - 1) / kColThreads;     // 3
+      int st_lds[kPer], st_chan[kPer], st_sp[kPer];
 #pragma unroll
-          for (int k = 1; k < kColWaves; ++k) w += (gi >= segstart[k]) ? 1 : 0;
-          const int a = s0 + s_idx[w][gi - segstart[w]];
-          const float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
-          const float radius = radii[a];
-          const float tf = floorf(type_index[a]) - (float)cbase;
-          const bool typed = tf >= 0.f && tf < (float)nchan;
-          float ar, ar2;
-          {
-#pragma clang fp contract(off)
-            ar = radius * g.radius_scale;
-            ar2 = ar * ar;
-          }
-          // an atom of another channel group (or an ignored one) can never hit
-          const float w4 = typed ? (BINARY ? ar2 : 1.0f / ar2) : (BINARY ? -1.0f : INFINITY);
-          s_rec[tid] = make_float4(ax, ay, az, w4);
-          s_rectype[tid] = typed ? (unsigned char)(int)tf : 0;
-          if (EXACT) {
-            const uint3 cl = pack_clip(g, ox, oy, oz, ax, ay, az, radius);
-            s_clip[tid] = make_uint4(cl.x, cl.y, cl.z, __float_as_uint(ar));
-          }
-        }
-        __syncthreads();
-
-        // ---- cull per 4x4x4 block, then splat ------------------------------------
+      for (int k = 0; k < kPer; ++k) {
+        const int item = tid + k * kColThreads;
+        const int j = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
+        const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
+        st_lds[k] = j * kPlane + row * kRowPad + f4 * 4;
+        st_chan[k] = (gx < dim && gy < dim && gz < dim) ? j : -1;
+        st_sp[k] = (gx * dim + gy) * dim + gz;
+      }
 #pragma unroll
-        for (int blk = 0; blk < kBlocksPerWave; ++blk) {
-          const int zb = z0 + (wave * kBlocksPerWave + blk) * 4;
-          if (zb >= zend) continue;
-          const float blz = grid_coord(oz, zb, g.resolution);
-          const float bhz = grid_coord(oz, min(zb + 4, zend) - 1, g.resolution);
-          const int vzi = zb + lz;
-          const bool live = xy_live && vzi < zend;
-          const float vz = grid_coord(oz, vzi, g.resolution);
-          for (int r0 = 0; r0 < m; r0 += kWave) {
-            const int i = r0 + lane;
-            bool pass = false;
-            float4 rec = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (i < m) {
-              rec = s_rec[i];
-              const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
-              pass = BINARY ? (d2 <= rec.w * kCullSlack) : (d2 * rec.w <= frm2 * kCullSlack);
-            }
-            const unsigned long long bm = __ballot(pass);
-            const int n = __popcll(bm);
-            if (n == 0) continue;
-            if (pass) {
-              const int p = __popcll(bm & ((1ull << lane) - 1ull));
-              s_mini[wave][p] = rec;
-              s_minitype[wave][p] = s_rectype[i];
-              if (EXACT) s_miniclip[wave][p] = s_clip[i];
-            }
-            const float4* mp = s_mini[wave];
-            const unsigned char* tp = s_minitype[wave];
-            auto body = [&](const float4& r, int tt, int it) {
-              const int t = __builtin_amdgcn_readfirstlane(tt);
-              bool inside = live;
-              float ar = 0.f;
-              if (EXACT) {
-                const uint4 cl = s_miniclip[wave][it];
-                inside = inside && inside_clip(vxi, vyi, vzi, make_uint3(cl.x, cl.y, cl.z));
-                ar = __uint_as_float(cl.w);
-              }
-              float val = density<BINARY, EXACT>(g, vx - r.x, vy - r.y, vz - r.z, r.w, ar, frm2, grm2);
-              if (!inside) val = 0.f;
-              // binary occupancy stores 1 where any atom covers the voxel
-              if (blk == 0) acc0[t] = BINARY ? fmaxf(acc0[t], val) : acc0[t] + val;
-              else if (blk == 1) acc1[t] = BINARY ? fmaxf(acc1[t], val) : acc1[t] + val;
-              else acc2[t] = BINARY ? fmaxf(acc2[t], val) : acc2[t] + val;
-            };
-            // software pipelined: the next record is in flight while this one is evaluated
-            float4 cur = mp[0];
-            int ct = tp[0];
-            int it = 0;
-            for (; it + 2 <= n; it += 2) {
-              const float4 r1 = mp[it + 1];
-              const int t1 = tp[it + 1];
-              body(cur, ct, it);
-              cur = mp[min(it + 2, kWave - 1)];
-              ct = tp[it + 2];
-              body(r1, t1, it + 1);
-            }
-            if (it < n) body(cur, ct, it);
+      for (int r = 0; r < (kRegChannels + kStageCh - 1) / kStageCh; ++r) {
+        if (r * kStageCh >= nchan) break;
+        float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
+#pragma unroll
+        for (int j = 0; j < kStageCh; ++j) {
+          const int c = r * kStageCh + j;
+          if (c < kRegChannels) {
+            stage[j * kPlane + dump_off] = MG_SUMS_AT(acc0, c);
+            stage[j * kPlane + dump_off + 4] = MG_SUMS_AT(acc1, c);
+            stage[j * kPlane + dump_off + 8] = MG_SUMS_AT(acc2, c);
           }
         }
         lds_barrier();
-      }
-    }
-
-    // ---- store: four channels per round through a double-buffered LDS stage ------
-    // fixed positions of this thread in the staged write-out (float4 granules)
-    constexpr int kItems = kStageCh * 16 * (kSlabZ / 4);               // 768 per round
-    constexpr int kPer = (kItems + kColThreads - 1) / kColThreads;     // 3
-    int st_lds[kPer], st_chan[kPer], st_sp[kPer];
+        float* ob = out_b + (size_t)(cbase + r * kStageCh) * chan_stride;
+        const int nch = min(kStageCh, nchan - r * kStageCh);
 #pragma unroll
-    for (int k = 0; k < kPer; ++k) {
-      const int item = tid + k * kColThreads;
-      const int j = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
-      const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
-      st_lds[k] = j * kPlane + row * kRowPad + f4 * 4;
-      st_chan[k] = (gx < dim && gy < dim && gz < dim) ? j : -1;
-      st_sp[k] = (gx * dim + gy) * dim + gz;
-    }
-#pragma unroll
-    for (int r = 0; r < (kRegChannels + kStageCh - 1) / kStageCh; ++r) {
-      if (r * kStageCh >= nchan) break;
-      float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
-#pragma unroll
-      for (int j = 0; j < kStageCh; ++j) {
-        const int c = r * kStageCh + j;
-        if (c < kRegChannels) {
-          stage[j * kPlane + dump_off] = acc0[c];
-          stage[j * kPlane + dump_off + 4] = acc1[c];
-          stage[j * kPlane + dump_off + 8] = acc2[c];
-        }
-      }
-      lds_barrier();
-      float* ob = out_b + (size_t)(cbase + r * kStageCh) * chan_stride;
-      const int nch = min(kStageCh, nchan - r * kStageCh);
-#pragma unroll
-      for (int k = 0; k < kPer; ++k) {
-        if (st_chan[k] >= 0 && st_chan[k] < nch) {
-          const v4f v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
-          float* dst = ob + (size_t)st_chan[k] * chan_stride + st_sp[k];
-          const int gz = z0 + ((tid + k * kColThreads) % 12) * 4;
-          if (vec_store && gz + 3 < dim) {
-            *reinterpret_cast<v4f*>(dst) = v;
-          } else {
-            dst[0] = v.x;
-            if (gz + 1 < dim) dst[1] = v.y;
-            if (gz + 2 < dim) dst[2] = v.z;
-            if (gz + 3 < dim) dst[3] = v.w;
+        for (int k = 0; k < kPer; ++k) {
+          if (st_chan[k] >= 0 && st_chan[k] < nch) {
+            const v4f v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
+            float* dst = ob + (size_t)st_chan[k] * chan_stride + st_sp[k];
+            const int gz = z0 + ((tid + k * kColThreads) % 12) * 4;
+            if ((vec_store & 1) && gz + 3 < dim) {
+              *reinterpret_cast<v4f*>(dst) = v;
+            } else {
+              dst[0] = v.x;
+              if (gz + 1 < dim) dst[1] = v.y;
+              if (gz + 2 < dim) dst[2] = v.z;
+              if (gz + 3 < dim) dst[3] = v.w;
+            }
           }
         }
       }
+      lds_barrier();
     }
-    lds_barrier();
   }
 }
 
-template <bool BINARY, bool EXACT>
+template <bool BINARY, bool EXACT, bool VEC>
 hipError_t launch_one(const GridArg& g, const BatchArg& batch, int nbatch, const Vec3Arg& centers,
-                      const float* coords, const float* type_index, const float* radii,
-                      float* out, hipStream_t stream) {
+                      const float* coords, const float* types, const float* radii, float* out,
+                      hipStream_t stream) {
   const int cols_per_side = (g.dim + kColXY - 1) / kColXY;
   const int slabs = (g.dim + kSlabZ - 1) / kSlabZ;
   const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
-  const int vec_store = (g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0) &&
-                        ((chan_stride * g.ntypes) % 4 == 0);
-  hipLaunchKernelGGL((splat_index_kernel<BINARY, EXACT>),
-                     dim3(cols_per_side * cols_per_side * slabs, nbatch), dim3(kColThreads), 0,
-                     stream, g, batch, centers, coords, type_index, radii, out, cols_per_side,
-                     vec_store);
+  // bit 0: float4 stores of the grid are aligned; bit 1: rows of the weight matrix are
+  int vec_store = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0) &&
+                   ((chan_stride * g.ntypes) % 4 == 0)) ? 1 : 0;
+  if (VEC && g.ntypes % 4 == 0 && (reinterpret_cast<uintptr_t>(types) & 15) == 0) vec_store |= 2;
+  const int groups = cols_per_side * ((cols_per_side + kColsPerGroup - 1) / kColsPerGroup);
+  hipLaunchKernelGGL((splat_column_kernel<BINARY, EXACT, VEC>),
+                     dim3(groups * slabs, nbatch), dim3(kColThreads), 0,
+                     stream, g, batch, centers, coords, types, radii, out, cols_per_side, vec_store);
   return hipGetLastError();
+}
+
+template <bool VEC>
+hipError_t launch_mode(const GridArg& g, const BatchArg& batch, int nbatch, const Vec3Arg& centers,
+                       const float* coords, const float* types, const float* radii, float* out,
+                       bool binary, bool exact, hipStream_t stream) {
+  if (binary && exact)
+    return launch_one<true, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+  if (binary)
+    return launch_one<true, false, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+  if (exact)
+    return launch_one<false, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+  return launch_one<false, false, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
 }
 
 }  // namespace
@@ -308,13 +439,16 @@ hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nba
                                 const Vec3Arg& centers, const float* coords,
                                 const float* type_index, const float* radii, float* out,
                                 bool binary, bool exact, hipStream_t stream) {
-  if (binary && exact)
-    return launch_one<true, true>(g, batch, nbatch, centers, coords, type_index, radii, out, stream);
-  if (binary)
-    return launch_one<true, false>(g, batch, nbatch, centers, coords, type_index, radii, out, stream);
-  if (exact)
-    return launch_one<false, true>(g, batch, nbatch, centers, coords, type_index, radii, out, stream);
-  return launch_one<false, false>(g, batch, nbatch, centers, coords, type_index, radii, out, stream);
+  return launch_mode<false>(g, batch, nbatch, centers, coords, type_index, radii, out, binary, exact,
+                            stream);
+}
+
+hipError_t launch_forward_vector_column(const GridArg& g, const BatchArg& batch, int nbatch,
+                                        const Vec3Arg& centers, const float* coords,
+                                        const float* type_vector, const float* radii, float* out,
+                                        bool binary, bool exact, hipStream_t stream) {
+  return launch_mode<true>(g, batch, nbatch, centers, coords, type_vector, radii, out, binary, exact,
+                           stream);
 }
 
 }  // namespace mg
