@@ -9,6 +9,9 @@ from ._capi import LIB_PATH, lib as _lib  # noqa: F401  (fails loudly if the .so
 from .gridding import (AtomBatch, CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
                        float3, set_random_seed, transform_batch)
 
+from .torch_bindings import (BatchedCoords2GridFunction, Coords2Grid, Coords2GridFunction,  # noqa: F401,E402
+                             Grid2CoordsGradientFunction)
+
 __version__ = "0.1.0"
 
 

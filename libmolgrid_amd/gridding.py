@@ -625,9 +625,11 @@ class GridMaker(object):
         a_out.finish()
 
     def _forward_padded(self, centers, coords, types, radii, grid):
-        # include/libmolgrid/grid_maker.h:265-301
-        a_centers = _Arg(centers, "centers", 2)
+        # include/libmolgrid/grid_maker.h:265-301; one centre for all examples is accepted too
+        one_center = not hasattr(centers, "shape") or len(tuple(centers.shape)) == 1
+        chost = _capi.f3(_to_float3(centers)) if one_center else _capi.f3(_Z3)
         a_coords = _Arg(coords, "coords", 3)
+        a_centers = _Shape((a_coords.shape[0], 3)) if one_center else _Arg(centers, "centers", 2)
         tdim = len(tuple(types.shape))
         if tdim not in (2, 3):
             raise ValueError("Unsupported types dimension")
@@ -650,8 +652,8 @@ class GridMaker(object):
             self._check_vector_args(n, _Shape(a_types.shape[1:]), _Shape(a_radii.shape[1:]),
                                     a_out.shape[1:])
             fn = _lib.mg_forward_vector
-        code = fn(self._p, B, None, n, a_centers.ptr, _capi.f3(_Z3), a_coords.ptr, a_types.ptr,
-                  a_radii.ptr, a_out.shape[1], a_out.ptr, _stream())
+        code = fn(self._p, B, None, n, None if one_center else a_centers.ptr, chost, a_coords.ptr,
+                  a_types.ptr, a_radii.ptr, a_out.shape[1], a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward")
         a_out.finish()
 
@@ -712,6 +714,8 @@ class GridMaker(object):
         if len(args) not in (6, 7):
             raise TypeError("backward expects 4 to 7 arguments")
         center, coords, types, radii, diff, agrad = args[:6]
+        if len(tuple(coords.shape)) == 3:
+            return self._backward_padded(*args)
         c = _to_float3(center)
         a_coords = _Arg(coords, "coords", 2)
         tdim = len(tuple(types.shape))
@@ -777,6 +781,66 @@ class GridMaker(object):
                 raise ValueError("diff does not have correct dimension %d: %d vs %d"
                                  % (ax, a_diff.shape[ax], dim))
         code = _lib.mg_backward_vector(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr,
+                                       a_types.ptr, a_radii.ptr, T, a_diff.ptr, a_ag.ptr,
+                                       a_tg.ptr, _stream())
+        _capi.check(code, "GridMaker.backward")
+        a_ag.finish()
+        a_tg.finish()
+
+    def _backward_padded(self, centers, coords, types, radii, diff, agrad, tgrad=None):
+        """Padded batch (B leading): coords (B,N,3), types (B,N) or (B,N,T), radii (B,N),
+        diff (B,T,D,D,D) -> gradients shaped like coords / types.  One launch for the batch.
+        ``centers`` is (B,3) or one centre for every example."""
+        a_coords = _Arg(coords, "coords", 3)
+        tdim = len(tuple(types.shape))
+        if tdim not in (2, 3):
+            raise ValueError("Unsupported types dimension")
+        a_types = _Arg(types, "types", tdim)
+        a_radii = _Arg(radii, "radii", 2)
+        a_diff = _Arg(diff, "diff", 5)
+        a_ag = _Arg(agrad, "atom_gradients", 3, out=True)
+        B, n = a_coords.shape[0], a_coords.shape[1]
+        for a in (a_types, a_radii, a_diff, a_ag):
+            if a.shape[0] != B:
+                raise ValueError("Mismatched batch sizes: %d vs %d" % (a.shape[0], B))
+        if a_ag.shape != a_coords.shape or a_coords.shape[2] != 3:
+            raise ValueError("Gradient dimension doesn't equal number of coordinates")
+        if a_types.shape[1] != n:
+            raise ValueError("Type dimension doesn't equal number of coordinates.")
+        dim = int(self._p.dim)
+        for ax in (2, 3, 4):
+            if a_diff.shape[ax] != dim:
+                raise ValueError("diff does not have correct dimension %d: %d vs %d"
+                                 % (ax - 1, a_diff.shape[ax], dim))
+        T = a_diff.shape[1]
+        one_center = not hasattr(centers, "shape") or len(tuple(centers.shape)) == 1
+        cen = None if one_center else _small_device(centers, 3)
+        chost = _capi.f3(_to_float3(centers)) if one_center else _capi.f3(_Z3)
+        if cen is not None and cen.shape[0] != B:
+            raise ValueError("Mismatched batch sizes: %d vs %d" % (cen.shape[0], B))
+        rti = bool(self._p.radii_type_indexed)
+        if tdim == 2:
+            if rti:
+                raise ValueError("Type indexed radii not supported with index types.")
+            if a_radii.shape[1] != n:
+                raise ValueError("Radii dimension doesn't equal number of coordinates")
+            code = _lib.mg_backward_index(self._p, B, None, n, _ptr(cen), chost, a_coords.ptr,
+                                          a_types.ptr, a_radii.ptr, T, a_diff.ptr, a_ag.ptr,
+                                          _stream())
+            _capi.check(code, "GridMaker.backward")
+            a_ag.finish()
+            return
+        if tgrad is None:
+            raise TypeError("vector types need a type_gradients argument")
+        a_tg = _Arg(tgrad, "type_gradients", 3, out=True)
+        if a_types.shape[2] != T:
+            raise ValueError("Channels in diff doesn't equal number of types")
+        if a_tg.shape != a_types.shape:
+            raise ValueError("Type gradient dimension has wrong number of types")
+        if a_radii.shape[1] != (T if rti else n):
+            raise ValueError("Radii dimension doesn't equal number of %s"
+                             % ("types" if rti else "coordinates"))
+        code = _lib.mg_backward_vector(self._p, B, None, n, _ptr(cen), chost, a_coords.ptr,
                                        a_types.ptr, a_radii.ptr, T, a_diff.ptr, a_ag.ptr,
                                        a_tg.ptr, _stream())
         _capi.check(code, "GridMaker.backward")
