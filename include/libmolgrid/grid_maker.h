@@ -143,15 +143,81 @@ class GridMaker {
     forward(in, t, out);
   }
 
-  /// batch of examples -> 5-D grid
+  /// batch of examples -> 5-D grid.  Index-typed examples are merged and packed on the host once,
+  /// uploaded once, and gridded with two launches for the whole batch (transform, splat); each
+  /// example gets its own random transformation about its own centre, as in the per-example call.
   template <typename Dtype, bool isCUDA>
   void forward(const std::vector<Example>& in, Grid<Dtype, 5, isCUDA>& out, float random_translation = 0.0,
                bool random_rotation = false) const {
+    require_float<Dtype>();
     if (in.size() != out.dimension(0))
       throw std::out_of_range("output grid dimension does not match size of example vector");
-    for (unsigned i = 0, n = in.size(); i < n; ++i) {
-      Grid<Dtype, 4, isCUDA> g(out[i]);
-      forward<Dtype, isCUDA>(in[i], g, random_translation, random_rotation);
+    const size_t B = in.size();
+    if (B == 0) return;
+    std::vector<CoordinateSet> merged(B);
+    bool packable = true;
+    size_t total = 0;
+    for (size_t i = 0; i < B; ++i) {
+      merged[i] = in[i].merge_coordinates();
+      if (merged[i].max_type != out.dimension(1))
+        throw std::out_of_range("Incorrect number of channels in output grid: " + itoa(merged[i].max_type) + " vs " + itoa(out.dimension(1)));
+      if (merged[i].has_vector_types() && merged[i].size() > 0) packable = false;
+      total += merged[i].size();
+    }
+    if (!packable || p.radii_type_indexed) {  // vector-typed sets: example by example
+      for (size_t i = 0; i < B; ++i) {
+        Grid<Dtype, 4, isCUDA> g(out[i]);
+        forward<Dtype, isCUDA>(in[i], g, random_translation, random_rotation);
+      }
+      return;
+    }
+    std::vector<float> coords(total * 3), types(total), radii(total), quats(B * 4), centers(B * 3), shifts(B * 3);
+    std::vector<int> offsets(B + 1, 0);
+    int longest = 1;
+    for (size_t i = 0, at = 0; i < B; ++i) {
+      const CoordinateSet& c = merged[i];
+      const size_t n = c.size();
+      float3 cen = make_float3(0, 0, 0);
+      for (int k = (int)in[i].sets.size() - 1; k >= 0; --k)
+        if (in[i].sets[k].size()) {
+          cen = in[i].sets.back().center();
+          break;
+        }
+      Transform t(cen, random_translation, random_rotation);
+      const Quaternion& q = t.get_quaternion();
+      const float3 tr = t.get_translation();
+      const float qv[4] = {q.R_component_1(), q.R_component_2(), q.R_component_3(), q.R_component_4()};
+      std::copy(qv, qv + 4, quats.begin() + 4 * i);
+      centers[3 * i] = cen.x, centers[3 * i + 1] = cen.y, centers[3 * i + 2] = cen.z;
+      shifts[3 * i] = tr.x, shifts[3 * i + 1] = tr.y, shifts[3 * i + 2] = tr.z;
+      if (n) {
+        std::copy(c.coords.cpu().data(), c.coords.cpu().data() + 3 * n, coords.begin() + 3 * at);
+        std::copy(c.type_index.cpu().data(), c.type_index.cpu().data() + n, types.begin() + at);
+        std::copy(c.radii.cpu().data(), c.radii.cpu().data() + n, radii.begin() + at);
+      }
+      at += n;
+      offsets[i + 1] = (int)at;
+      longest = std::max(longest, (int)n);
+    }
+    detail::DeviceStaging<float> dc(coords.data(), coords.size()), dt(types.data(), total), dr(radii.data(), total);
+    detail::DeviceStaging<float> dq(quats.data(), quats.size()), dcen(centers.data(), centers.size()), dsh(shifts.data(), shifts.size());
+    detail::DeviceStaging<int> doff(offsets.data(), offsets.size());
+    const float zero3[3] = {0, 0, 0}, ident[4] = {1, 0, 0, 0};
+    if (total)
+      abi_check(mg_transform_forward((int)B, doff.get(), longest, dq.get(), ident, dcen.get(), zero3, dsh.get(), zero3,
+                                     1, dc.get(), dc.get(), nullptr),
+                "GridMaker::forward");
+    if (isCUDA) {
+      abi_check(mg_forward_index(&p, (int)B, doff.get(), longest, dcen.get(), zero3, dc.get(), dt.get(), dr.get(),
+                                 (int)out.dimension(1), reinterpret_cast<float*>(out.data()), nullptr),
+                "GridMaker::forward");
+      LMG_HIP_CHECK(hipDeviceSynchronize());  // the staged inputs are released on return
+    } else {
+      detail::DeviceStaging<float> dout(out.size());
+      abi_check(mg_forward_index(&p, (int)B, doff.get(), longest, dcen.get(), zero3, dc.get(), dt.get(), dr.get(),
+                                 (int)out.dimension(1), dout.get(), nullptr),
+                "GridMaker::forward");
+      dout.download(reinterpret_cast<float*>(out.data()));
     }
   }
 

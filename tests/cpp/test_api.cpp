@@ -195,6 +195,27 @@ static void gpu_tests() {
   g1.forward(ex, Transform(), eg.gpu());
   CHECK(eg(2, 16, 12, 12) > 0.99f);   // ligand atom at (1,0,0) lands in channel 2
   CHECK(throws<std::out_of_range>([&] { MGrid4f wrong(2, 25, 25, 25); g1.forward(ex, Transform(), wrong.gpu()); }));
+
+  // batch of examples: one packed upload, two launches; equals the per-example calls bit for bit
+  Example ex2;
+  ex2.sets.push_back(CoordinateSet(p1, std::vector<int>{1}, std::vector<float>{2.0f}, 2));
+  ex2.sets.push_back(CoordinateSet(two, std::vector<int>{0, 0}, std::vector<float>{1, 1.5f}, 1));
+  Example none;
+  none.sets.push_back(CoordinateSet(std::vector<float3>{}, std::vector<int>{}, std::vector<float>{}, 2));
+  none.sets.push_back(CoordinateSet(std::vector<float3>{}, std::vector<int>{}, std::vector<float>{}, 1));
+  std::vector<Example> batch{ex, ex2, none};
+  MGrid5f bg(3, 3, 25, 25, 25), bh(3, 3, 25, 25, 25);
+  g1.forward(batch, bg.gpu());
+  g1.forward(batch, bh.cpu());
+  bg.tocpu();
+  CHECK(std::memcmp(bg.cpu().data(), bh.cpu().data(), bg.size() * sizeof(float)) == 0);
+  for (int b = 0; b < 3; ++b) {
+    MGrid4f one(3, 25, 25, 25);
+    g1.forward(batch[b], one.gpu());
+    one.tocpu();
+    CHECK(std::memcmp(one.cpu().data(), bg.cpu().data() + (size_t)b * one.size(), one.size() * sizeof(float)) == 0);
+  }
+  CHECK(throws<std::out_of_range>([&] { MGrid5f wrong(2, 3, 25, 25, 25); g1.forward(batch, wrong.gpu()); }));
 }
 
 int main(int argc, char** argv) {

@@ -73,6 +73,6 @@ def test_module_optimises_coordinates(mg):
         loss.backward()
         opt.step()
         first = first if first is not None else float(loss.detach())
-    assert float(loss) < 0.05 * first
+    assert float(loss.detach()) < 0.05 * first
     assert np.allclose(coords.detach().cpu().numpy(), [[1.0, 0.5, -0.5]], atol=0.1)
     assert "resolution 0.50" in repr(layer)
