@@ -43,6 +43,7 @@ constexpr int kStageCh = 4;                      // channels staged per round
 constexpr int kSuper = 4096;                     // atoms scanned per pass
 constexpr int kSeg = kSuper / kColWaves;         // per wave
 constexpr int kRecChunk = 256;
+constexpr int kPairBytes = 48;                   // two records and their tags in a block's list
 
 // A float that is the same in every lane, moved to a scalar register so that it does not occupy
 // a vector register for the whole kernel.
@@ -50,21 +51,81 @@ __device__ __forceinline__ float uniform(float v) {
   return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
 }
 
-// The 28 channel sums of one voxel are addressed with a wave-uniform channel index, which the
-// compiler turns into scalar-indexed register moves.  Register tuples come in sizes 16 and 12 (not
-// 28), so each voxel keeps two plain arrays (lo: channels 0-15, hi: 16-27) selected by a scalar
-// branch: 28 registers where one array of 28 would take 32.
-constexpr int kLoChannels = 16;
-constexpr int kHiChannels = kRegChannels - kLoChannels;
-#define MG_SUMS_DECL(name) float name##_lo[kLoChannels], name##_hi[kHiChannels]
-#define MG_SUMS_AT(name, c) ((c) < kLoChannels ? name##_lo[(c) < kLoChannels ? (c) : 0] \
-                                               : name##_hi[(c) < kLoChannels ? 0 : (c) - kLoChannels])
+// The channel sums -- 28 per voxel, three voxels (blocks) per lane -- are kept in registers that
+// the compiler does not know about: it is limited to v0 .. v(MG_ACC_BASE-1) by the kernel's
+// amdgpu_num_vgpr attribute, and the 84 registers from v(MG_ACC_BASE) on are touched only by the
+// asm statements below, through the scalar register index (s_set_gpr_idx).  One indexed VALU
+// instruction adds a density to the sum of (block, channel); with a C array the compiler spends
+// three moves and, for arrays that are not a register-tuple size, copies of the whole array.
+// The build checks the generated code: no compiler-allocated register may reach the reserved range.
+#define MG_ACC_BASE 84
+#define MG_ACC_TOP "v167"
+constexpr int kAccRegs = kBlocksPerWave * kRegChannels;
+static_assert(MG_ACC_BASE + kAccRegs - 1 == 167, "MG_ACC_TOP names the last reserved register");
 
+// sum[idx] (+)= val; idx is wave-uniform
 template <bool BINARY>
-__device__ __forceinline__ void sums_add(float (&lo)[kLoChannels], float (&hi)[kHiChannels], int t,
-                                         float val) {
-  if (t < kLoChannels) lo[t] = BINARY ? fmaxf(lo[t], val) : lo[t] + val;
-  else hi[t - kLoChannels] = BINARY ? fmaxf(hi[t - kLoChannels], val) : hi[t - kLoChannels] + val;
+__device__ __forceinline__ void acc_add(int idx, float val) {
+  if (BINARY)
+    asm volatile("s_set_gpr_idx_on %1, gpr_idx(SRC0,DST)\n\tv_max_f32 v[%2], v[%2], %0\n\ts_set_gpr_idx_off"
+                 :: "v"(val), "s"(idx), "n"(MG_ACC_BASE) : MG_ACC_TOP);
+  else
+    asm volatile("s_set_gpr_idx_on %1, gpr_idx(SRC0,DST)\n\tv_add_f32 v[%2], v[%2], %0\n\ts_set_gpr_idx_off"
+                 :: "v"(val), "s"(idx), "n"(MG_ACC_BASE) : MG_ACC_TOP);
+}
+// all sums = 0
+#define MG_XSTR2(x) #x
+#define MG_XSTR(x) MG_XSTR2(x)
+#define MG_Z1(e) "v_mov_b32 v[" MG_XSTR(MG_ACC_BASE) "+" #e "], 0\n\t"
+#define MG_Z4(e) MG_Z1(e+0) MG_Z1(e+1) MG_Z1(e+2) MG_Z1(e+3)
+#define MG_Z28(e) MG_Z4(e+0) MG_Z4(e+4) MG_Z4(e+8) MG_Z4(e+12) MG_Z4(e+16) MG_Z4(e+20) MG_Z4(e+24)
+__device__ __forceinline__ void acc_zero_all() {
+  static_assert(kAccRegs == 84, "the list below clears 3 x 28 registers");
+  asm volatile(MG_Z28(0) MG_Z28(28) MG_Z28(56) "s_nop 0" ::: MG_ACC_TOP);
+}
+// Channels 4R .. 4R+3 of the lane's three voxels -> the LDS stage.  `a0`, `a1`, `a2` are the LDS
+// byte addresses of the three voxels in plane 0 of stage buffer 0; planes are 13 x 256 bytes
+// apart and the two stage buffers 52 x 256 bytes, which the 256-byte-granular offsets of
+// ds_write2st64_b32 reach, so one instruction writes two channels.
+template <int R>
+__device__ __forceinline__ void acc_dump_round(unsigned a0, unsigned a1, unsigned a2) {
+  static_assert(kPlane * 4 == 13 * 256 && kStageCh == 4, "offsets below");
+  constexpr int buf = (R & 1) * 52;
+  asm volatile("ds_write2st64_b32 %0, v[%3], v[%3+1] offset0:%4 offset1:%5\n\t"
+               "ds_write2st64_b32 %0, v[%3+2], v[%3+3] offset0:%6 offset1:%7\n\t"
+               "ds_write2st64_b32 %1, v[%3+28], v[%3+29] offset0:%4 offset1:%5\n\t"
+               "ds_write2st64_b32 %1, v[%3+30], v[%3+31] offset0:%6 offset1:%7\n\t"
+               "ds_write2st64_b32 %2, v[%3+56], v[%3+57] offset0:%4 offset1:%5\n\t"
+               "ds_write2st64_b32 %2, v[%3+58], v[%3+59] offset0:%6 offset1:%7"
+               :: "v"(a0), "v"(a1), "v"(a2), "n"(MG_ACC_BASE + 4 * R), "n"(buf), "n"(buf + 13),
+                  "n"(buf + 26), "n"(buf + 39)
+               : "memory", MG_ACC_TOP);
+}
+
+// sums[first + c] += val * w[c] for seven channels starting at the compile-time channel C0;
+// first (= block * 28) is wave-uniform, the weights are scalars
+template <int C0>
+__device__ __forceinline__ void acc_fma7(int first, float val, float w0, float w1, float w2, float w3,
+                                         float w4, float w5, float w6) {
+  asm volatile("s_set_gpr_idx_on %1, gpr_idx(SRC2,DST)\n\t"
+               "v_fma_f32 v[%9], %2, %0, v[%9]\n\t"
+               "v_fma_f32 v[%10], %3, %0, v[%10]\n\t"
+               "v_fma_f32 v[%11], %4, %0, v[%11]\n\t"
+               "v_fma_f32 v[%12], %5, %0, v[%12]\n\t"
+               "v_fma_f32 v[%13], %6, %0, v[%13]\n\t"
+               "v_fma_f32 v[%14], %7, %0, v[%14]\n\t"
+               "v_fma_f32 v[%15], %8, %0, v[%15]\n\t"
+               "s_set_gpr_idx_off"
+               :: "v"(val), "s"(first), "s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4), "s"(w5), "s"(w6),
+                  "n"(MG_ACC_BASE + C0), "n"(MG_ACC_BASE + C0 + 1), "n"(MG_ACC_BASE + C0 + 2),
+                  "n"(MG_ACC_BASE + C0 + 3), "n"(MG_ACC_BASE + C0 + 4), "n"(MG_ACC_BASE + C0 + 5),
+                  "n"(MG_ACC_BASE + C0 + 6)
+               : MG_ACC_TOP);
+}
+
+// byte address of a __shared__ object inside the workgroup's LDS
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  return (unsigned)(unsigned long)(const __attribute__((address_space(3))) void*)p;
 }
 
 // LDS-only barrier: outstanding global stores are not waited for.
@@ -74,7 +135,7 @@ __device__ __forceinline__ void lds_barrier() {
 
 // `types` is type_index [n] (VEC = false) or type_vector [n, ntypes] (VEC = true)
 template <bool BINARY, bool EXACT, bool VEC>
-__global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) void splat_column_kernel(
+__global__ __launch_bounds__(kColThreads) void splat_column_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ types, const float* __restrict__ radii,
     float* __restrict__ out, int cols_per_side, int vec_store) {
@@ -84,10 +145,11 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
   __shared__ unsigned char s_rectype[VEC ? 1 : kRecChunk];   // channel of the record (index types)
   __shared__ int s_recatom[VEC ? kRecChunk : 1];             // atom of the record (vector types)
   __shared__ uint4 s_clip[EXACT ? kRecChunk : 1];  // index box + ar, EXACT only
-  __shared__ float4 s_mini[kColWaves][kWave];
+  // wave-private list of a block's atoms, two per 48-byte entry: records at +0 and +16, then
+  // their channels (two bytes at +32) or atom numbers (two ints at +32, VEC); two spare entries
+  // because the splat loop reads ahead
+  __shared__ __align__(16) unsigned char s_mini[kColWaves][(kWave / 2 + 2) * kPairBytes];
   __shared__ uint4 s_miniclip[EXACT ? kColWaves : 1][EXACT ? kWave : 1];
-  __shared__ unsigned char s_minitype[VEC ? 1 : kColWaves][VEC ? 1 : kWave + 4];
-  __shared__ int s_miniatom[VEC ? kColWaves : 1][VEC ? kWave + 4 : 1];
   __shared__ __align__(16) float s_stage[2 * kStageCh * kPlane];
 
   const int tid = threadIdx.x;
@@ -123,6 +185,8 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
   const float gly = uniform(grid_coord(oy, gy0, g.resolution));
   const float ghy = uniform(grid_coord(oy, min(gy0 + kColXY * kColsPerGroup, dim) - 1, g.resolution));
 
+  float quad_c = g.C;                       // constant term of the quadratic tail, kept in a
+  asm volatile("" : "+v"(quad_c));          // vector register (an fma takes one scalar operand)
   const float frm2 = uniform(g.frm * g.frm);
   const float grm2 = uniform(g.grm * g.grm);
   const float cull_mult = BINARY ? 1.0f : g.frm;  // support radius / ar
@@ -237,13 +301,7 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
       const float cly = uniform(grid_coord(oy, y0, g.resolution));
       const float chy = uniform(grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution));
 
-      MG_SUMS_DECL(acc0);
-      MG_SUMS_DECL(acc1);
-      MG_SUMS_DECL(acc2);
-#pragma unroll
-      for (int c = 0; c < kLoChannels; ++c) acc0_lo[c] = acc1_lo[c] = acc2_lo[c] = 0.f;
-#pragma unroll
-      for (int c = 0; c < kHiChannels; ++c) acc0_hi[c] = acc1_hi[c] = acc2_hi[c] = 0.f;
+      acc_zero_all();
 
       for (int s0 = begin; s0 < end; s0 += pass_len) {
         if (!one_pass) scan(s0, min(end, s0 + kSuper));
@@ -252,7 +310,7 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
           if (!records_cached) build_records(s0, c0, m, cbase, nchan);
 
           // ---- cull per 4x4x4 block, then splat ----------------------------------
-#pragma unroll
+#pragma unroll 1
           for (int blk = 0; blk < kBlocksPerWave; ++blk) {
             const int zb = z0 + (wave * kBlocksPerWave + blk) * 4;
             if (zb >= zend) continue;
@@ -260,7 +318,9 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
             const float bhz = uniform(grid_coord(oz, min(zb + 4, zend) - 1, g.resolution));
             const int vzi = zb + lz;
             const bool live = xy_live && vzi < zend;
-            const float vz = grid_coord(oz, vzi, g.resolution);
+            // a voxel outside the grid sits at infinity: no atom reaches it
+            const float vz = live ? grid_coord(oz, vzi, g.resolution) : INFINITY;
+            const int acc0 = blk * kRegChannels;
             for (int r0 = 0; r0 < m; r0 += kWave) {
               const int i = r0 + lane;
               bool pass = false;
@@ -273,28 +333,32 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
               const unsigned long long bm = __ballot(pass);
               const int n = __popcll(bm);
               if (n == 0) continue;
+              unsigned char* mine = s_mini[wave];
               if (pass) {
                 const int p = __popcll(bm & ((1ull << lane) - 1ull));
-                s_mini[wave][p] = rec;
-                if (VEC) s_miniatom[wave][p] = s_recatom[i];
-                else s_minitype[wave][p] = s_rectype[i];
+                unsigned char* e = mine + (p >> 1) * kPairBytes;
+                *reinterpret_cast<float4*>(e + (p & 1) * 16) = rec;
+                if (VEC) *reinterpret_cast<int*>(e + 32 + (p & 1) * 4) = s_recatom[i];
+                else e[32 + (p & 1)] = s_rectype[i];
                 if (EXACT) s_miniclip[wave][p] = s_clip[i];
               }
-              const float4* mp = s_mini[wave];
-              auto tag = [&](int k) -> int { return VEC ? s_miniatom[wave][k] : (int)s_minitype[wave][k]; };
-              auto body = [&](const float4& r, int tt, int it) {
-                const int t = __builtin_amdgcn_readfirstlane(tt);   // channel, or atom (VEC)
-                bool inside = live;
+              // one atom of the list against this lane's voxel; the sum is touched only where
+              // the atom reaches the voxel
+              auto splat = [&](const float4& r, int tag, int it) {
                 float ar = 0.f;
+                bool inside = true;
                 if (EXACT) {
                   const uint4 cl = s_miniclip[wave][it];
-                  inside = inside && inside_clip(vxi, vyi, vzi, make_uint3(cl.x, cl.y, cl.z));
+                  inside = inside_clip(vxi, vyi, vzi, make_uint3(cl.x, cl.y, cl.z));
                   ar = __uint_as_float(cl.w);
                 }
-                float val = density<BINARY, EXACT>(g, vx - r.x, vy - r.y, vz - r.z, r.w, ar, frm2, grm2);
-                if (!inside) val = 0.f;
-                if (VEC) {
-                  const float* __restrict__ tv = types + (size_t)t * g.ntypes + cbase;
+                float val;
+                const bool hit = density_hit<BINARY, EXACT>(g, vx - r.x, vy - r.y, vz - r.z, r.w, ar,
+                                                            frm2, grm2, quad_c, val);
+                if (!VEC) {
+                  if (hit && inside) acc_add<BINARY>(acc0 + tag, val);
+                } else {
+                  const float* __restrict__ tv = types + (size_t)tag * g.ntypes + cbase;
                   // the atom's weights, through wave-uniform loads issued together
                   float wgt[kRegChannels];
                   if (full_group && (vec_store & 2)) {   // 16-byte aligned rows: seven 4-wide loads
@@ -311,39 +375,46 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
 #pragma unroll
                     for (int c = 0; c < kRegChannels; ++c) wgt[c] = c < nchan ? tv[c] : 0.f;
                   }
-                  auto weigh = [&](float (&lo)[kLoChannels], float (&hi)[kHiChannels]) {
-#pragma unroll
-                    for (int c = 0; c < kRegChannels; ++c) {
-                      float& sum = c < kLoChannels ? lo[c < kLoChannels ? c : 0]
-                                                   : hi[c < kLoChannels ? 0 : c - kLoChannels];
-                      // binary occupancy adds the weight itself where the atom covers the voxel
-                      if (BINARY) sum += (val != 0.f) ? wgt[c] : 0.f;
-                      else sum = fmaf(val, wgt[c], sum);
-                    }
-                  };
-                  if (blk == 0) weigh(acc0_lo, acc0_hi);
-                  else if (blk == 1) weigh(acc1_lo, acc1_hi);
-                  else weigh(acc2_lo, acc2_hi);
-                } else {
-                  // binary occupancy stores 1 where any atom covers the voxel
-                  if (blk == 0) sums_add<BINARY>(acc0_lo, acc0_hi, t, val);
-                  else if (blk == 1) sums_add<BINARY>(acc1_lo, acc1_hi, t, val);
-                  else sums_add<BINARY>(acc2_lo, acc2_hi, t, val);
+                  if (hit && inside) {
+                    // binary occupancy (val is 1) adds the weight itself: fma(w, 1, sum) = sum + w
+                    acc_fma7<0>(acc0, val, wgt[0], wgt[1], wgt[2], wgt[3], wgt[4], wgt[5], wgt[6]);
+                    acc_fma7<7>(acc0, val, wgt[7], wgt[8], wgt[9], wgt[10], wgt[11], wgt[12], wgt[13]);
+                    acc_fma7<14>(acc0, val, wgt[14], wgt[15], wgt[16], wgt[17], wgt[18], wgt[19], wgt[20]);
+                    acc_fma7<21>(acc0, val, wgt[21], wgt[22], wgt[23], wgt[24], wgt[25], wgt[26], wgt[27]);
+                  }
                 }
               };
-              // software pipelined: the next record is in flight while this one is evaluated
-              float4 cur = mp[0];
-              int ct = tag(0);
-              int it = 0;
-              for (; it + 2 <= n; it += 2) {
-                const float4 r1 = mp[it + 1];
-                const int t1 = tag(it + 1);
-                body(cur, ct, it);
-                cur = mp[min(it + 2, kWave - 1)];
-                ct = tag(it + 2);
-                body(r1, t1, it + 1);
+              struct Pair { float4 r0, r1; int t0, t1; };
+              auto fetch = [&](int k) -> Pair {
+                const unsigned char* e = mine + k * kPairBytes;
+                Pair q;
+                q.r0 = *reinterpret_cast<const float4*>(e);
+                q.r1 = *reinterpret_cast<const float4*>(e + 16);
+                if (VEC) {
+                  q.t0 = *reinterpret_cast<const int*>(e + 32);
+                  q.t1 = *reinterpret_cast<const int*>(e + 36);
+                } else {
+                  q.t0 = *reinterpret_cast<const unsigned short*>(e + 32);
+                  q.t1 = 0;
+                }
+                return q;
+              };
+              auto splat_pair = [&](const Pair& q, int it) {
+                int t0 = __builtin_amdgcn_readfirstlane(q.t0), t1;
+                if (VEC) t1 = __builtin_amdgcn_readfirstlane(q.t1);
+                else { t1 = t0 >> 8; t0 &= 0xff; }
+                splat(q.r0, t0, it);
+                if (it + 1 < n) splat(q.r1, t1, it + 1);
+              };
+              // four atoms per trip; entry k+1 is in flight while entry k is evaluated
+              Pair pa = fetch(0);
+              for (int it = 0; it < n; it += 4) {
+                const Pair pb = fetch((it >> 1) + 1);
+                splat_pair(pa, it);
+                if (it + 2 >= n) break;
+                pa = fetch((it >> 1) + 2);
+                splat_pair(pb, it + 2);
               }
-              if (it < n) body(cur, ct, it);
             }
           }
           if (!records_cached) lds_barrier();   // records are rebuilt next round
@@ -364,19 +435,10 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
         st_chan[k] = (gx < dim && gy < dim && gz < dim) ? j : -1;
         st_sp[k] = (gx * dim + gy) * dim + gz;
       }
-#pragma unroll
-      for (int r = 0; r < (kRegChannels + kStageCh - 1) / kStageCh; ++r) {
-        if (r * kStageCh >= nchan) break;
-        float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
-#pragma unroll
-        for (int j = 0; j < kStageCh; ++j) {
-          const int c = r * kStageCh + j;
-          if (c < kRegChannels) {
-            stage[j * kPlane + dump_off] = MG_SUMS_AT(acc0, c);
-            stage[j * kPlane + dump_off + 4] = MG_SUMS_AT(acc1, c);
-            stage[j * kPlane + dump_off + 8] = MG_SUMS_AT(acc2, c);
-          }
-        }
+      const unsigned dump0 = lds_address(s_stage + dump_off);
+      const unsigned dump1 = dump0 + 16, dump2 = dump0 + 32;
+      auto store_round = [&](int r) {
+        const float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
         lds_barrier();
         float* ob = out_b + (size_t)(cbase + r * kStageCh) * chan_stride;
         const int nch = min(kStageCh, nchan - r * kStageCh);
@@ -396,7 +458,15 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_num_vgpr(168))) 
             }
           }
         }
-      }
+      };
+      static_assert(kRegChannels == 7 * kStageCh, "seven rounds below");
+      acc_dump_round<0>(dump0, dump1, dump2); store_round(0);
+      if (nchan > 4) { acc_dump_round<1>(dump0, dump1, dump2); store_round(1); }
+      if (nchan > 8) { acc_dump_round<2>(dump0, dump1, dump2); store_round(2); }
+      if (nchan > 12) { acc_dump_round<3>(dump0, dump1, dump2); store_round(3); }
+      if (nchan > 16) { acc_dump_round<4>(dump0, dump1, dump2); store_round(4); }
+      if (nchan > 20) { acc_dump_round<5>(dump0, dump1, dump2); store_round(5); }
+      if (nchan > 24) { acc_dump_round<6>(dump0, dump1, dump2); store_round(6); }
       lds_barrier();
     }
   }
@@ -424,12 +494,17 @@ template <bool VEC>
 hipError_t launch_mode(const GridArg& g, const BatchArg& batch, int nbatch, const Vec3Arg& centers,
                        const float* coords, const float* types, const float* radii, float* out,
                        bool binary, bool exact, hipStream_t stream) {
-  if (binary && exact)
-    return launch_one<true, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+  if constexpr (!VEC) {
+    if (binary && exact)
+      return launch_one<true, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+    if (exact)
+      return launch_one<false, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
+  } else {
+    // vector types with the exact predicates are not instantiated here (register budget)
+    if (exact) return hipErrorInvalidValue;
+  }
   if (binary)
     return launch_one<true, false, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
-  if (exact)
-    return launch_one<false, true, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
   return launch_one<false, false, VEC>(g, batch, nbatch, centers, coords, types, radii, out, stream);
 }
 

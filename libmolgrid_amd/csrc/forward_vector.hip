@@ -261,8 +261,9 @@ hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nb
                                  const float* type_vector, const float* radii, float* out,
                                  bool binary, bool radii_type_indexed, bool exact,
                                  hipStream_t stream) {
-  // per-atom radii take the column kernel; only type-indexed radii use the cubic-tile kernel below
-  if (!radii_type_indexed)
+  // per-atom radii take the column kernel; type-indexed radii and the exact-predicate modes
+  // (truncated Gaussian) use the cubic-tile kernel below
+  if (!radii_type_indexed && !exact)
     return launch_forward_vector_column(g, batch, nbatch, centers, coords, type_vector, radii, out,
                                         binary, exact, stream);
   if (binary && radii_type_indexed)

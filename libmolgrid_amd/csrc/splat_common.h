@@ -176,6 +176,30 @@ __device__ __forceinline__ float density(const GridArg& g, float dx, float dy, f
   }
 }
 
+// The same density split into "does the atom reach the voxel" (returned) and the value where it
+// does, so that callers can leave untouched sums alone.  `quad_c` is g.C (in a vector register).
+template <bool BINARY, bool EXACT>
+__device__ __forceinline__ bool density_hit(const GridArg& g, float dx, float dy, float dz, float w,
+                                            float ar, float frm2, float grm2, float quad_c,
+                                            float& val) {
+  if (BINARY) {
+    const float rsq = sq_distance_exact(dx, dy, dz);
+    val = 1.0f;
+    return rsq < w;
+  } else if (EXACT) {
+    val = density<false, true>(g, dx, dy, dz, w, ar, frm2, grm2);
+    return val != 0.f;
+  } else {
+    const float rsq = dx * dx + dy * dy + dz * dz;
+    const float u = rsq * w;
+    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+    const float su = __builtin_amdgcn_sqrtf(u);
+    const float quad = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+    val = (u <= grm2) ? gauss : quad;
+    return u <= frm2;
+  }
+}
+
 }  // namespace mg
 
 #endif

@@ -40,6 +40,25 @@ def test_forward_small_vs_oracle(mg, ntypes, binary):
         assert_close(out.cpu().numpy(), ref, what="vector forward")
 
 
+@pytest.mark.parametrize("gm_args", [
+    (0.5, 11.5, False, False, 1.0, -1.5),   # truncated Gaussian, no quadratic tail
+    (0.5, 11.5, True, False, 1.0, -0.5),    # binary sphere wider than its index box
+    (0.5, 11.5, False, False, 1.3, 0.7),    # radius scale + early quadratic
+])
+def test_forward_unusual_radius_multiples(mg, gm_args):
+    """The modes that evaluate the reference's own cut-off predicates, with vector types."""
+    rng = np.random.default_rng(11)
+    coords, tv, radii = make_case(rng, 70, 5, 7.0)
+    ref = oracle.GridMaker(*gm_args).forward((0, 0.1, 0), coords, tv, radii)
+    gm = mg.GridMaker(*gm_args)
+    out = torch.full(gm.grid_dimensions(5), -1.0, device="cuda")
+    gm.forward((0, 0.1, 0), dev(coords), dev(tv), dev(radii), out)
+    if gm_args[2]:
+        assert np.array_equal(out.cpu().numpy(), ref)
+    else:
+        assert_close(out.cpu().numpy(), ref, what="vector forward, exact predicates")
+
+
 @pytest.mark.parametrize("binary", [False, True])
 def test_forward_type_indexed_radii(mg, binary):
     rng = np.random.default_rng(7)
