@@ -1,8 +1,8 @@
 // Atom-gradient (and type-gradient) accumulation on gfx950.
 //
 // One wavefront owns one atom: its 64 lanes sweep the atom's voxel box
-// (src/grid_maker.cu:66-79) in a fixed lane -> voxel order, each lane keeps a
-// private partial sum, and the partials are combined with a DPP reduction tree
+// (src/grid_maker.cu:66-79) -- every lane marches along x through one (y, z) column of the box --
+// each lane keeps a private partial sum, and the partials are combined with a DPP reduction tree
 // inside the wave.  No global float atomics are used, so the result is
 // reproducible run to run.  Per-voxel terms follow accumulate_atom_gradient and
 // density_grad_dist (src/grid_maker.cu:881-919); the CPU loops being mirrored
@@ -43,59 +43,101 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-// Lane-strided walk over a box of ni*nj*nk voxels, k fastest: lane L visits
-// linear indices L, L+64, L+128, ...  The mixed-radix step of 64 is worked out
-// once per box so that the inner loop needs no division.
-struct BoxWalk {
-  int i, j, k;     // current offset inside the box
-  int off;         // linear element offset of the current voxel inside one grid channel
-  int di, dj, dk;  // 64 expressed in (nj*nk, nk, 1) digits
-  int nj, nk;
-  int step;        // offset advance of one stride when no digit wraps
-  int wrap_k, wrap_j;  // offset corrections when k / j wrap
-  // box origin (lo0, lo1, lo2) inside a dim^3 channel
-  __device__ __forceinline__ void start(int lane, int nj_, int nk_, int lo0, int lo1, int lo2,
-                                        int dim) {
-    nj = nj_;
-    nk = nk_;
-    const int plane = nj * nk;
-    i = lane / plane;
-    int r = lane - i * plane;
-    j = r / nk;
-    k = r - j * nk;
-    di = kWave / plane;
-    r = kWave - di * plane;
-    dj = r / nk;
-    dk = r - dj * nk;
-    off = ((lo0 + i) * dim + lo1 + j) * dim + lo2 + k;
-    step = (di * dim + dj) * dim + dk;
-    wrap_k = dim - nk;             // k -= nk, ++j
-    wrap_j = (dim - nj) * dim;     // j -= nj, ++i
+// Sweep of an atom's voxel box [lo, lo+n) by one wave.  Each lane owns one (y, z) column of the
+// box (64 columns per pass) and marches along x, so everything that depends on y and z only --
+// dy, dz, dy^2+dz^2, the lane's element offset -- is worked out once per pass, while the x offset
+// of a plane is the same in every lane: it is computed by lane i for plane i before the march
+// and read back as a scalar.  body(dx, dy, dz, dist2, plane_off, lane_off, live) is called for
+// every voxel; dx and plane_off (element offset of the plane) are wave-uniform, lane_off is the
+// lane's element offset inside the plane, and lanes past the last column get live = false and an
+// infinite dist2 (their offsets point at a valid voxel of the box).
+template <typename Body>
+__device__ __forceinline__ void sweep_box(const GridArg& g, int lane, float ox, float oy, float oz,
+                                          float ax, float ay, float az, int lo0, int lo1, int lo2,
+                                          int ni, int nj, int nk, Body body) {
+  const int dim = g.dim;
+  const int columns = nj * nk;
+  for (int i0 = 0; i0 < ni; i0 += kWave) {
+    const int planes = min(kWave, ni - i0);
+    const int dx_lane = __float_as_int(grid_coord(ox, lo0 + i0 + lane, g.resolution) - ax);
+    for (int c0 = 0; c0 < columns; c0 += kWave) {
+      const bool live = c0 + lane < columns;
+      const int c = live ? c0 + lane : columns - 1;
+      const int j = c / nk, k = c - j * nk;
+      const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+      const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+      const float dyz2 = live ? dy * dy + dz * dz : INFINITY;
+      const unsigned lane_off = (unsigned)((lo1 + j) * dim + lo2 + k);
+      for (int i = 0; i < planes; ++i) {
+        const float dx = __int_as_float(__builtin_amdgcn_readlane(dx_lane, i));
+        const unsigned plane_off = (unsigned)(lo0 + i0 + i) * (unsigned)(dim * dim);
+        body(dx, dy, dz, fmaf(dx, dx, dyz2), plane_off, lane_off, live);
+      }
+    }
   }
-  __device__ __forceinline__ void next() {
-    k += dk;
-    off += step;
-    if (k >= nk) { k -= nk; ++j; off += wrap_k; }
-    j += dj;
-    if (j >= nj) { j -= nj; ++i; off += wrap_j; }
-    i += di;
+}
+
+// sweep_box for callers that read one float per voxel from `chan` (one grid channel): the reads
+// of kSweepChunk planes are issued together before any of them is used, so that a wave has
+// several planes in flight instead of one round trip to memory per voxel.
+constexpr int kSweepChunk = 8;
+template <typename Body>
+__device__ __forceinline__ void sweep_channel(const GridArg& g, const float* __restrict__ chan,
+                                              int lane, float ox, float oy, float oz, float ax,
+                                              float ay, float az, int lo0, int lo1, int lo2, int ni,
+                                              int nj, int nk, Body body) {
+  const int dim = g.dim;
+  const int columns = nj * nk;
+  const unsigned plane_stride = (unsigned)(dim * dim);
+  for (int i0 = 0; i0 < ni; i0 += kWave) {
+    const int planes = min(kWave, ni - i0);
+    const int dx_lane = __float_as_int(grid_coord(ox, lo0 + i0 + lane, g.resolution) - ax);
+    for (int c0 = 0; c0 < columns; c0 += kWave) {
+      const bool live = c0 + lane < columns;
+      const int c = live ? c0 + lane : columns - 1;
+      const int j = c / nk, k = c - j * nk;
+      const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+      const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+      const float dyz2 = live ? dy * dy + dz * dz : INFINITY;
+      const unsigned lane_off = (unsigned)((lo1 + j) * dim + lo2 + k);
+      for (int i = 0; i < planes; i += kSweepChunk) {
+        const float* first = chan + (size_t)(unsigned)(lo0 + i0 + i) * plane_stride;
+        float gv[kSweepChunk];
+#pragma unroll
+        for (int u = 0; u < kSweepChunk; ++u)
+          if (i + u < planes) gv[u] = (first + (size_t)u * plane_stride)[lane_off];
+#pragma unroll
+        for (int u = 0; u < kSweepChunk; ++u) {
+          if (i + u < planes) {
+            const float dx = __int_as_float(__builtin_amdgcn_readlane(dx_lane, i + u));
+            body(dx, dy, dz, fmaf(dx, dx, dyz2), gv[u], live);
+          }
+        }
+      }
+    }
   }
-};
+}
 
 // Per-atom constants of the gradient scale.
 struct GradConsts {
   float inv_ar2;   // 1/ar^2
+  float exp_k;     // -2 log2(e) / ar^2  (exp(-2u) = exp2(exp_k * dist^2))
   float gauss;     // 4/ar^2            (Gaussian part:  scale = gauss * exp(-2u) * gridval)
   float quad_a;    // -D/ar^2           (quadratic part: scale = (quad_a + quad_b/dist) * gridval)
   float quad_b;    // -E/ar
+  float core2;     // (grm ar)^2: dist^2 up to here is Gaussian
+  float reach2;    // (frm ar)^2: dist^2 beyond is untouched
 };
 __device__ __forceinline__ GradConsts grad_consts(const GridArg& g, float ar) {
   GradConsts c;
   const float inv_ar = 1.0f / ar;
   c.inv_ar2 = inv_ar * inv_ar;
+  c.exp_k = c.inv_ar2 * kNeg2Log2e;
   c.gauss = 4.0f * c.inv_ar2;
   c.quad_a = -g.D * c.inv_ar2;
   c.quad_b = -g.E * inv_ar;
+  c.core2 = g.grm * g.grm * ar * ar;
+  c.reach2 = g.frm * g.frm * ar * ar;
   return c;
 }
 
@@ -105,13 +147,13 @@ __device__ __forceinline__ GradConsts grad_consts(const GridArg& g, float ar) {
 //   Gaussian, u <= grm^2:  d/d(dist) = -4 dist/ar^2 exp(-2u)   ->  4/ar^2 exp(-2u) gridval
 //   quadratic tail:        d/d(dist) = (D dist/ar + E)/ar      -> -(D/ar^2 + E/(ar dist)) gridval
 // and 0 where the reference skips the voxel (dist == 0 or beyond the cut-off).
-__device__ __forceinline__ float grad_scale(const GradConsts& c, float dist2, float frm2,
-                                            float grm2, float gridval) {
-  const float u = dist2 * c.inv_ar2;
-  const float e = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+__device__ __forceinline__ float grad_scale(const GradConsts& c, float dist2, float gridval) {
+  const float e = __builtin_amdgcn_exp2f(dist2 * c.exp_k);
   const float rinv = __builtin_amdgcn_rsqf(dist2);
-  const float s = (u <= grm2) ? c.gauss * e : fmaf(c.quad_b, rinv, c.quad_a);
-  return (dist2 > 0.f && u <= frm2) ? s * gridval : 0.f;
+  const float s = (dist2 <= c.core2) ? c.gauss * e : fmaf(c.quad_b, rinv, c.quad_a);
+  // dist2 == 0 (which the reference skips) needs no test: it lies in the Gaussian core, where s is
+  // finite, and the caller multiplies the result by a zero offset
+  return (dist2 <= c.reach2) ? s * gridval : 0.f;
 }
 
 template <bool BINARY>
@@ -125,7 +167,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
     const float* __restrict__ type_index, const float* __restrict__ radii,
     const float* __restrict__ diff, float* __restrict__ atom_gradients) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so is the atom
   const int b = blockIdx.y;
   int begin, end;
   example_range(batch, b, begin, end);
@@ -136,7 +178,6 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
   const int dim = g.dim;
   const size_t chan_stride = (size_t)dim * dim * dim;
   const float* diff_b = diff + (size_t)b * g.ntypes * chan_stride;
-  const float frm2 = g.frm * g.frm, grm2 = g.grm * g.grm;
 
   for (int a = begin + blockIdx.x * kBwdWaves + wave; a < end; a += gridDim.x * kBwdWaves) {
     float gx = 0.f, gy = 0.f, gz = 0.f;
@@ -157,22 +198,14 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
       bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
       const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
       if (ni > 0 && nj > 0 && nk > 0) {
-        const char* chan = reinterpret_cast<const char*>(diff_b + (size_t)(int)tf * chan_stride);
-        BoxWalk w;
-        w.start(lane, nj, nk, lo0, lo1, lo2, dim);
-        for (; w.i < ni; w.next()) {
-          const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
-          const float dx = grid_coord(ox, xi, g.resolution) - ax;
-          const float dy = grid_coord(oy, yi, g.resolution) - ay;
-          const float dz = grid_coord(oz, zi, g.resolution) - az;
-          const float dist2 = dx * dx + dy * dy + dz * dz;
-          // one channel of the grid is < 4 GiB: a 32-bit byte offset from the uniform base
-          const float gv = *reinterpret_cast<const float*>(chan + (unsigned)w.off * 4u);
-          const float sc = grad_scale(gc, dist2, frm2, grm2, gv);
-          gx = fmaf(dx, sc, gx);
-          gy = fmaf(dy, sc, gy);
-          gz = fmaf(dz, sc, gz);
-        }
+        const float* chan = diff_b + (size_t)(int)tf * chan_stride;
+        sweep_channel(g, chan, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
+                      [&](float dx, float dy, float dz, float dist2, float gv, bool) {
+                        const float sc = grad_scale(gc, dist2, gv);
+                        gx = fmaf(dx, sc, gx);
+                        gy = fmaf(dy, sc, gy);
+                        gz = fmaf(dz, sc, gz);
+                      });
       }
     }
     gx = wave_sum(gx);
@@ -195,7 +228,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
     const float* __restrict__ diff, float* __restrict__ atom_gradients,
     float* __restrict__ type_gradients) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so is the atom
   const int b = blockIdx.y;
   int begin, end;
   example_range(batch, b, begin, end);
@@ -239,30 +272,27 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
 #pragma unroll
         for (int t = 0; t < TG; ++t) tg[t] = 0.f;
         if (any) {
-          BoxWalk w;
-          w.start(lane, nj, nk, lo0, lo1, lo2, dim);
-          for (; w.i < ni; w.next()) {
-            const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
-            const float dx = grid_coord(ox, xi, g.resolution) - ax;
-            const float dy = grid_coord(oy, yi, g.resolution) - ay;
-            const float dz = grid_coord(oz, zi, g.resolution) - az;
-            const float dist2 = dx * dx + dy * dy + dz * dz;
-            const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
-            const float* p = diff_b + (size_t)cbase * chan_stride + w.off;
-            float weighted = 0.f;  // sum_t weight_t * diff_t at this voxel
+          const float* group = diff_b + (size_t)cbase * chan_stride;
+          sweep_box(g, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
+                    [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
+                        unsigned lane_off, bool live) {
+                      float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+                      if (!live) val = 0.f;
+                      const float* p = group + plane_off;
+                      float weighted = 0.f;  // sum_t weight_t * diff_t at this voxel
 #pragma unroll
-            for (int t = 0; t < TG; ++t) {
-              if (t < nchan) {
-                const float gv = p[(size_t)t * chan_stride];
-                tg[t] = fmaf(val, gv, tg[t]);
-                weighted = fmaf(tv[cbase + t], gv, weighted);
-              }
-            }
-            const float sc = grad_scale(gc, dist2, frm2, grm2, weighted);
-            gx = fmaf(dx, sc, gx);
-            gy = fmaf(dy, sc, gy);
-            gz = fmaf(dz, sc, gz);
-          }
+                      for (int t = 0; t < TG; ++t) {
+                        if (t < nchan) {
+                          const float gv = (p + (size_t)t * chan_stride)[lane_off];
+                          tg[t] = fmaf(val, gv, tg[t]);
+                          weighted = fmaf(tv[cbase + t], gv, weighted);
+                        }
+                      }
+                      const float sc = grad_scale(gc, dist2, weighted);
+                      gx = fmaf(dx, sc, gx);
+                      gy = fmaf(dy, sc, gy);
+                      gz = fmaf(dz, sc, gz);
+                    });
         }
 #pragma unroll
         for (int t = 0; t < TG; ++t) {
@@ -294,22 +324,16 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         float tgt = 0.f, tx = 0.f, ty = 0.f, tz = 0.f;
         if (ni > 0 && nj > 0 && nk > 0) {
           const float* chan = diff_b + (size_t)t * chan_stride;
-          BoxWalk w;
-          w.start(lane, nj, nk, lo0, lo1, lo2, dim);
-          for (; w.i < ni; w.next()) {
-            const int xi = lo0 + w.i, yi = lo1 + w.j, zi = lo2 + w.k;
-            const float dx = grid_coord(ox, xi, g.resolution) - ax;
-            const float dy = grid_coord(oy, yi, g.resolution) - ay;
-            const float dz = grid_coord(oz, zi, g.resolution) - az;
-            const float dist2 = dx * dx + dy * dy + dz * dz;
-            const float gv = chan[w.off];
-            const float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
-            tgt = fmaf(val, gv, tgt);
-            const float sc = grad_scale(gc, dist2, frm2, grm2, gv);
-            tx = fmaf(dx, sc, tx);
-            ty = fmaf(dy, sc, ty);
-            tz = fmaf(dz, sc, tz);
-          }
+          sweep_channel(g, chan, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
+                        [&](float dx, float dy, float dz, float dist2, float gv, bool live) {
+                          float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+                          if (!live) val = 0.f;
+                          tgt = fmaf(val, gv, tgt);
+                          const float sc = grad_scale(gc, dist2, gv);
+                          tx = fmaf(dx, sc, tx);
+                          ty = fmaf(dy, sc, ty);
+                          tz = fmaf(dz, sc, tz);
+                        });
         }
         const float s = wave_sum(tgt);
         if (lane == 0) type_gradients[(size_t)a * T + t] = s;
