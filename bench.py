@@ -90,6 +90,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the four launches of a step as one captured HIP graph (measured: "
+                         "no faster than launching them one by one, which is the default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU (examples are independent; a larger job "
@@ -145,12 +148,31 @@ def main():
         k_backward()
         k_unrotate()
 
-    for _ in range(args.warmup):
+    run_step = step
+    if args.graph:
+        # the four launches of a step as one HIP graph: nothing in them allocates or synchronises
         step()
+        torch.cuda.synchronize()
+        eager = (grid.clone(), grads.clone())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(2):          # replays must reproduce the eager results bit for bit
+            grid.zero_()
+            grads.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            if not (torch.equal(grid, eager[0]) and torch.equal(grads, eager[1])):
+                raise RuntimeError("HIP graph replay differs from the eager step")
+        del eager
+        run_step = graph.replay
+
+    for _ in range(args.warmup):
+        run_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
@@ -169,13 +191,13 @@ def main():
 
     dominant_fwd = ms_fwd >= ms_bwd
     roofline = {
-        "kernel": "splat_index_kernel (forward)" if dominant_fwd else "backward_index_kernel",
+        "kernel": "splat_column_kernel (forward)" if dominant_fwd else "backward_index_kernel",
         "bound": "hbm",
         "achieved": round(fwd_gbs if dominant_fwd else bwd_gbs, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
-        "traffic": measured_traffic("splat_index_kernel" if dominant_fwd
+        "traffic": measured_traffic("splat_column_kernel" if dominant_fwd
                                     else "backward_index_kernel"),
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
@@ -222,6 +244,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "launch": "hip graph replay" if args.graph else "eager",
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
