@@ -148,6 +148,32 @@ class GridMaker:
                   _p(radii), ctypes.c_int64(ntypes), _p(diff), gp(agrad), gp(tgrad)))
         return agrad, tgrad
 
+    def backward_relevance(self, center, coords, types, radii, density, diff):
+        c = _f32(center)
+        coords, types, radii, density, diff = (_f32(coords), _f32(types), _f32(radii),
+                                               _f32(density), _f32(diff))
+        n = coords.shape[0]
+        rel = np.empty(n, np.float32)
+        _check(lib().orc_backward_relevance(
+            ctypes.byref(self.p), _p(c), ctypes.c_int64(n), _p(coords), _p(types), _p(radii),
+            ctypes.c_int64(diff.shape[0]), _p(density), _p(diff), _p(rel)))
+        return rel
+
+    def backward_gradients(self, center, coords, types, radii, diff, atom_gradients,
+                           type_gradients):
+        """-> (diffdiff, atom_diffdiff, type_diffdiff)"""
+        c = _f32(center)
+        coords, types, radii, diff = _f32(coords), _f32(types), _f32(radii), _f32(diff)
+        ag, tg = _f32(atom_gradients), _f32(type_gradients)
+        n, ntypes = coords.shape[0], diff.shape[0]
+        dd = np.empty(diff.shape, np.float32)
+        add = np.empty((n, 3), np.float32)
+        tdd = np.empty((n, ntypes), np.float32)
+        _check(lib().orc_backward_gradients(
+            ctypes.byref(self.p), _p(c), ctypes.c_int64(n), _p(coords), _p(types), _p(radii),
+            ctypes.c_int64(ntypes), _p(diff), _p(ag), _p(tg), _p(dd), _p(add), _p(tdd)))
+        return dd, add, tdd
+
     # -- packed batch -------------------------------------------------------
     def forward_batch(self, offsets, centers, coords, types, radii, ntypes, nthreads=1):
         off = np.ascontiguousarray(offsets, dtype=np.int64)

@@ -411,6 +411,166 @@ int orc_backward_vector_f64(const orc_gridmaker* g, const float center[3], int64
   return ORC_OK;
 }
 
+/* ---- relevance and second-order gradients -------------------------------- */
+
+/* src/grid_maker.cpp:392-432 (calc_atom_relevance_cpu) and :680-704 (backward_relevance):
+ * every voxel the atom reaches hands the atom the share val/density of its relevance. */
+int orc_backward_relevance(const orc_gridmaker* g, const float center[3], int64_t natoms,
+                           const float* coords, const float* type_index, const float* radii,
+                           int64_t ntypes, const float* density, const float* diff,
+                           float* relevance) {
+  memset(relevance, 0, (size_t)natoms * sizeof(float));
+  float origin[3];
+  grid_origin(g, center, origin);
+  const size_t chan = (size_t)g->dim * g->dim * g->dim;
+  const int64_t dim = g->dim;
+  for (int64_t a = 0; a < natoms; ++a) {
+    int which = (int)roundf(type_index[a]);
+    if (which < 0) continue;
+    if (which >= ntypes) return ORC_ERR_TYPE_RANGE;
+    const float* dens = density + (size_t)which * chan;
+    const float* dif = diff + (size_t)which * chan;
+    float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
+    float radius = radii[a];
+    float r = radius * g->radius_scale * g->final_radius_multiple;
+    unsigned lo[3], hi[3];
+    orc_bounds_1d(g, origin[0], ax, r, &lo[0], &hi[0]);
+    orc_bounds_1d(g, origin[1], ay, r, &lo[1], &hi[1]);
+    orc_bounds_1d(g, origin[2], az, r, &lo[2], &hi[2]);
+    float ret = 0;
+    for (size_t i = lo[0]; i < hi[0]; ++i)
+      for (size_t j = lo[1]; j < hi[1]; ++j)
+        for (size_t k = lo[2]; k < hi[2]; ++k) {
+          float x = origin[0] + i * g->resolution;
+          float y = origin[1] + j * g->resolution;
+          float z = origin[2] + k * g->resolution;
+          float val = orc_calc_point(g, ax, ay, az, radius, x, y, z);
+          if (val > 0) {
+            float denseval = dens[(i * dim + j) * dim + k];
+            float gridval = dif[(i * dim + j) * dim + k];
+            if (denseval > 0) ret += gridval * val / denseval;
+          }
+        }
+    relevance[a] = ret;
+  }
+  return ORC_OK;
+}
+
+/* src/grid_maker.cu:812-855: type_grad_grad and atom_density_grad_grad hold the same
+ * expression -- the derivative of -(a-x)/dist * density_grad_dist with respect to a. */
+static float density_grad_grad(const orc_gridmaker* g, float a, float x, float dist, float r) {
+  float dist2 = dist * dist;
+  if (dist > r * g->final_radius_multiple) return 0;
+  if (dist <= r * g->gaussian_radius_multiple) {
+    float r2 = r * r;
+    float ex = (float)(-2.0 * dist2 / r2);
+    return 16 * (a - x) * (a - x) * expf(ex) / (r2 * r2) - 4 * expf(ex) / (r2);
+  }
+  float ax = a - x;
+  float ax2 = ax * ax;
+  float term1 = (float)(-(g->E + g->D * dist / r) * ax2 / (pow(dist2, 1.5) * r));
+  float term2 = g->D * ax2 / (dist2 * r * r);
+  float term3 = (g->E + g->D * dist / r) / (dist * r);
+  return term1 + term2 + term3;
+}
+
+/* src/grid_maker.cu:858-877 (atom_density_grad_grad_other): mixed second derivative */
+static float density_grad_grad_other(const orc_gridmaker* g, float a, float x, float b, float y,
+                                     float dist, float r) {
+  float dist2 = dist * dist;
+  if (dist > r * g->final_radius_multiple) return 0;
+  if (dist <= r * g->gaussian_radius_multiple) {
+    float r2 = r * r;
+    float ex = (float)(-2.0 * dist2 / r2);
+    return 16 * (a - x) * (b - y) * expf(ex) / (r2 * r2);
+  }
+  float ax = a - x;
+  float by = b - y;
+  float term1 = (float)(-(g->E + g->D * dist / r) * ax * by / (pow(dist2, 1.5) * r));
+  float term2 = g->D * ax * by / (dist2 * r * r);
+  return term1 + term2;
+}
+
+/* src/grid_maker.cpp:529-661 (backward_gradients, CPU): gradients of the backward pass
+ * (atom_gradients, type_gradients as functions of coords, types and diff) with respect to
+ * diff (diffdiff), the coordinates (atom_diffdiff) and the types (type_diffdiff, zero). */
+int orc_backward_gradients(const orc_gridmaker* g, const float center[3], int64_t natoms,
+                           const float* coords, const float* type_vector, const float* radii,
+                           int64_t ntypes, const float* diff, const float* atom_gradients,
+                           const float* type_gradients, float* diffdiff, float* atom_diffdiff,
+                           float* type_diffdiff) {
+  if (g->binary) return ORC_ERR_ARGUMENT;
+  const size_t chan = (size_t)g->dim * g->dim * g->dim;
+  const int64_t dim = g->dim;
+  memset(atom_diffdiff, 0, (size_t)natoms * 3 * sizeof(float));
+  memset(type_diffdiff, 0, (size_t)natoms * ntypes * sizeof(float));
+  memset(diffdiff, 0, chan * ntypes * sizeof(float));
+  float origin[3];
+  grid_origin(g, center, origin);
+  for (int64_t a = 0; a < natoms; ++a) {
+    for (int64_t t = 0; t < ntypes; ++t) {
+      float tmult = type_vector[a * ntypes + t];
+      if (tmult == 0) continue;
+      const float* diffG = diff + (size_t)t * chan;
+      float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
+      float gx = atom_gradients[3 * a], gy = atom_gradients[3 * a + 1], gz = atom_gradients[3 * a + 2];
+      float tgrad = type_gradients[a * ntypes + t];
+      float radius = g->radii_type_indexed ? radii[t] : radii[a];
+      float ar = radius * g->radius_scale;
+      float densityrad = radius * g->radius_scale * g->final_radius_multiple;
+      unsigned lo[3], hi[3];
+      orc_bounds_1d(g, origin[0], ax, densityrad, &lo[0], &hi[0]);
+      orc_bounds_1d(g, origin[1], ay, densityrad, &lo[1], &hi[1]);
+      orc_bounds_1d(g, origin[2], az, densityrad, &lo[2], &hi[2]);
+      float dd[3] = {0, 0, 0};
+      for (size_t i = lo[0]; i < hi[0]; ++i)
+        for (size_t j = lo[1]; j < hi[1]; ++j)
+          for (size_t k = lo[2]; k < hi[2]; ++k) {
+            float x = origin[0] + i * g->resolution;
+            float y = origin[1] + j * g->resolution;
+            float z = origin[2] + k * g->resolution;
+            size_t off = (size_t)(i * dim + j) * dim + k;
+            float G = diffG[off];
+            float dist_x = x - ax, dist_y = y - ay, dist_z = z - az;
+            float dist2 = dist_x * dist_x + dist_y * dist_y + dist_z * dist_z;
+            double dist = sqrtf(dist2);
+            float agrad_dist = density_grad_dist(g, (float)dist, ar);
+            if (!isfinite(agrad_dist)) continue;
+            float gval = 0.0f;
+            if (dist > 0) {
+              gval += (float)(-(dist_x / dist) * (agrad_dist * gx));
+              gval += (float)(-(dist_y / dist) * (agrad_dist * gy));
+              gval += (float)(-(dist_z / dist) * (agrad_dist * gz));
+              gval *= tmult;
+            }
+            float val = orc_calc_point(g, ax, ay, az, radius, x, y, z);
+            gval += val * tgrad;
+            diffdiff[(size_t)t * chan + off] += gval;
+
+            float d = (float)dist;
+            dd[0] += density_grad_grad(g, ax, x, d, ar) * G * tmult * gx;
+            dd[0] += density_grad_grad_other(g, ax, x, ay, y, d, ar) * G * tmult * gy;
+            dd[0] += density_grad_grad_other(g, ax, x, az, z, d, ar) * G * tmult * gz;
+            dd[0] += density_grad_grad(g, ax, x, d, ar) * G * tgrad;
+
+            dd[1] += density_grad_grad_other(g, ay, y, ax, x, d, ar) * G * tmult * gx;
+            dd[1] += density_grad_grad(g, ay, y, d, ar) * G * tmult * gy;
+            dd[1] += density_grad_grad_other(g, ay, y, az, z, d, ar) * G * tmult * gz;
+            dd[1] += density_grad_grad(g, ay, y, d, ar) * G * tgrad;
+
+            dd[2] += density_grad_grad_other(g, az, z, ax, x, d, ar) * G * tmult * gx;
+            dd[2] += density_grad_grad_other(g, az, z, ay, y, d, ar) * G * tmult * gy;
+            dd[2] += density_grad_grad(g, az, z, d, ar) * G * tmult * gz;
+            dd[2] += density_grad_grad(g, az, z, d, ar) * G * tgrad;
+          }
+      atom_diffdiff[3 * a + 0] += dd[0];
+      atom_diffdiff[3 * a + 1] += dd[1];
+      atom_diffdiff[3 * a + 2] += dd[2];
+    }
+  }
+  return ORC_OK;
+}
+
 /* ---- quaternion / transform --------------------------------------------- */
 
 /* include/libmolgrid/quaternion.h:82-91 (Hamilton product, left-to-right sums) */

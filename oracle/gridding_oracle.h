@@ -100,6 +100,20 @@ int orc_backward_vector_f64(const orc_gridmaker* g, const float center[3], int64
                             int64_t ntypes, const float* diff, double* atom_gradients,
                             double* type_gradients);
 
+/* relevance of each atom (src/grid_maker.cpp:392-432, 680-704); density is the forward grid */
+int orc_backward_relevance(const orc_gridmaker* g, const float center[3], int64_t natoms,
+                           const float* coords, const float* type_index, const float* radii,
+                           int64_t ntypes, const float* density, const float* diff,
+                           float* relevance);
+
+/* gradients of the vector-typed backward pass (src/grid_maker.cpp:529-661); the three outputs
+ * are overwritten */
+int orc_backward_gradients(const orc_gridmaker* g, const float center[3], int64_t natoms,
+                           const float* coords, const float* type_vector, const float* radii,
+                           int64_t ntypes, const float* diff, const float* atom_gradients,
+                           const float* type_gradients, float* diffdiff, float* atom_diffdiff,
+                           float* type_diffdiff);
+
 /* quaternion stored as (a, b, c, d) = real, i, j, k */
 void orc_quat_mul(const float p[4], const float q[4], float out[4]);
 void orc_quat_inverse(const float q[4], float out[4]);

@@ -271,6 +271,133 @@ def test_vector_backward_linearity_and_type_gradient():
     assert np.array_equal(a1, a2) and np.array_equal(t1, t2)
 
 
+# ------------------------------------------- relevance, second-order pass ---
+def test_relevance_known_case_and_brute_force():
+    """test/test_gridmaker.cpp:313-337: one atom, one voxel with density 1 and relevance 10."""
+    g = oracle.GridMaker(0.1, 6.0)
+    d = g.dim
+    diff = np.zeros((1, d, d, d), np.float32)
+    dens = np.zeros((1, d, d, d), np.float32)
+    diff[0, 31, 30, 30] = 10.0
+    dens[0, 31, 30, 30] = 1.0
+    rel = g.backward_relevance((0, 0, 0), [[0, 0, 0]], [0], [2.0], dens, diff)
+    assert 1.0 < rel[0] < 10.0
+    assert rel[0] == pytest.approx(10.0 * np.exp(-2 * 0.1 ** 2 / 4.0), rel=1e-6)
+    # brute force over every voxel: sum diff * own density / total density where both are positive
+    rng = np.random.default_rng(21)
+    n, T = 12, 3
+    coords = rng.uniform(-3, 3, (n, 3)).astype(np.float32)
+    types = rng.integers(0, T, n).astype(np.float32)
+    types[3] = -1
+    radii = rng.uniform(1.0, 2.0, n).astype(np.float32)
+    for binary in (False, True):
+        gm = oracle.GridMaker(0.5, 9.5, binary)
+        total = gm.forward((0.1, 0, -0.2), coords, types, radii, T)
+        if binary:
+            total = total * rng.uniform(0.5, 2.0, total.shape).astype(np.float32)
+        total[0, 5:8] = 0           # voxels without density hand nothing on
+        diff = rng.standard_normal(total.shape).astype(np.float32)
+        rel = gm.backward_relevance((0.1, 0, -0.2), coords, types, radii, total, diff)
+        for a in range(n):
+            if types[a] < 0:
+                assert rel[a] == 0
+                continue
+            t = int(types[a])
+            own = gm.forward((0.1, 0, -0.2), coords[a:a + 1], [0], radii[a:a + 1], 1)[0]
+            ok = (own > 0) & (total[t] > 0)
+            want = (diff[t][ok].astype(np.float64) * own[ok] / total[t][ok]).sum()
+            assert rel[a] == pytest.approx(want, rel=1e-4, abs=1e-4)
+
+
+def test_backward_gradients_closed_form():
+    """test/test_gridmaker.py:439-466: d/dx of |d(density at one voxel)/dcoords|^2 for a full
+    Gaussian (multiple -2, radius 1) is -128 d^3 exp(-4 d^2) + 32 d exp(-4 d^2), d = x - 1."""
+    g = oracle.GridMaker(0.5, 6.0, gaussian_radius_multiple=-2.0)
+    types = np.ones((1, 1), np.float32)
+    radii = np.ones(1, np.float32)
+    for axis in range(3):
+        idx = [0, 6, 6, 6]
+        idx[1 + axis] = 8                   # the voxel at +1.0 on this axis
+        diff = np.zeros(g.grid_shape(1), np.float32)
+        diff[tuple(idx)] = 1.0
+        for x in np.arange(-0.9, 3, 0.1):
+            coords = np.zeros((1, 3), np.float32)
+            coords[0, axis] = x
+            lg, _ = g.backward((0, 0, 0), coords, types, radii, diff)
+            # fancyL = sum(lg^2): its gradient wrt lg is 2 lg, wrt the type gradient 0
+            dd, add, tdd = g.backward_gradients((0, 0, 0), coords, types, radii, diff, 2 * lg,
+                                                np.zeros((1, 1), np.float32))
+            d = float(coords[0, axis]) - 1
+            want = -128 * d ** 3 * np.exp(-4 * d ** 2) + 32 * d * np.exp(-4 * d ** 2)
+            assert add[0, axis] == pytest.approx(want, abs=1e-4)
+            assert not tdd.any()
+
+
+def test_backward_gradients_are_derivatives_of_backward():
+    """F(coords, diff) = <w, atom_gradients> + <v, type_gradients>: diffdiff = dF/ddiff (F is
+    linear in diff), type_diffdiff = 0, and, for v = 0, atom_diffdiff = dF/dcoords (central
+    differences of the double-accumulating backward pass).  The reference's v term of
+    atom_diffdiff is v * sum(diff * d2(density)/da2) (src/grid_maker.cpp:631, the same
+    expression as the coordinate term, src/grid_maker.cu:812-855), which is not dF/dcoords; it is
+    checked against the analytic second derivative of a pure Gaussian below."""
+    rng = np.random.default_rng(22)
+    n, T = 5, 2
+    coords = rng.uniform(-1.5, 1.5, (n, 3)).astype(np.float32)
+    tv = rng.uniform(0.2, 1, (n, T)).astype(np.float32)
+    tv[1, 0] = 0
+    radii = rng.uniform(1.2, 1.8, n).astype(np.float32)
+    g = oracle.GridMaker(0.25, 8.0)
+    ax = np.linspace(-1, 1, g.dim)
+    X, Y, Z = np.meshgrid(ax, ax, ax, indexing="ij")
+    diff = np.stack([np.sin(2 * X) + Y * Z, np.cos(3 * Y) - X * Z]).astype(np.float32)
+    w = rng.standard_normal((n, 3)).astype(np.float32)
+    v = rng.standard_normal((n, T)).astype(np.float32)
+
+    def F(c, dif):
+        ag, tg = g.backward((0, 0, 0), c, tv, radii, dif, f64=True)
+        # like the reference, a channel with zero weight takes no part in the second pass
+        return float((w * ag).sum() + (v * tg * (tv != 0)).sum())
+
+    dd, add, tdd = g.backward_gradients((0, 0, 0), coords, tv, radii, diff, w, v)
+    assert not tdd.any()
+    zero = np.zeros_like(v)
+    add = g.backward_gradients((0, 0, 0), coords, tv, radii, diff, w, zero)[1]
+    v_saved, v = v, zero
+    h = 2e-3
+    fd = np.zeros((n, 3))
+    for a in range(n):
+        for k in range(3):
+            cp, cm = coords.copy(), coords.copy()
+            cp[a, k] += h
+            cm[a, k] -= h
+            fd[a, k] = (F(cp, diff) - F(cm, diff)) / (float(cp[a, k]) - float(cm[a, k]))
+    # every component is a sum of hundreds of terms of either sign: compare on the scale of the sums
+    assert np.abs(add - fd).max() < 3e-3 * np.abs(fd).max()
+    v = v_saved
+    delta = rng.standard_normal(diff.shape).astype(np.float32)
+    lin = F(coords, diff + delta) - F(coords, diff)
+    assert float((dd.astype(np.float64) * delta).sum()) == pytest.approx(lin, rel=1e-3, abs=1e-3)
+    with pytest.raises(oracle.OracleError):
+        oracle.GridMaker(0.5, 6.0, True).backward_gradients((0, 0, 0), coords, tv, radii,
+                                                            np.zeros((T, 13, 13, 13), np.float32), w, v)
+    # the type-gradient term alone, pure Gaussian out to 2 r: v * sum(diff * d2/da2 exp(-2 d^2/r^2))
+    gg = oracle.GridMaker(0.25, 8.0, gaussian_radius_multiple=-2.0)
+    c1 = np.asarray([[0.3, -0.2, 0.1]], np.float32)
+    r1 = np.asarray([1.3], np.float32)
+    one = np.ones((1, 1), np.float32)
+    d1 = diff[:1]
+    got = gg.backward_gradients((0, 0, 0), c1, one, r1, d1, np.zeros((1, 3), np.float32),
+                                np.full((1, 1), 0.7, np.float32))[1]
+    pos = (-4.0 + 0.25 * np.arange(gg.dim)).astype(np.float64)
+    PX, PY, PZ = np.meshgrid(pos, pos, pos, indexing="ij")
+    rel = np.stack([PX - 0.3, PY + 0.2, PZ - 0.1])
+    d2 = (rel ** 2).sum(axis=0)
+    e = np.exp(-2 * d2 / 1.3 ** 2) * (np.sqrt(d2) <= 2 * 1.3)
+    for k in range(3):
+        second = (16 * rel[k] ** 2 / 1.3 ** 4 - 4 / 1.3 ** 2) * e
+        assert got[0, k] == pytest.approx(0.7 * (second * d1[0]).sum(), rel=2e-3, abs=2e-3)
+
+
 # ------------------------------------------------- quaternion / transform ---
 def test_quaternion_hamilton_rules():
     i, j, k = [0, 1, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1]
