@@ -415,7 +415,157 @@ class GridMaker {
     dtg.download(reinterpret_cast<float*>(type_gradients.data()));
   }
 
+  // ---- relevance (include/libmolgrid/grid_maker.h:547-618 of the reference) ----------------
+  /// index types, device arrays
+  template <typename Dtype>
+  void backward_relevance(float3 grid_center, const Grid<float, 2, true>& coords,
+                          const Grid<float, 1, true>& type_index, const Grid<float, 1, true>& radii,
+                          const Grid<Dtype, 4, true>& density, const Grid<Dtype, 4, true>& diff,
+                          Grid<Dtype, 1, true>& relevance) const {
+    require_float<Dtype>();
+    check_relevance(coords, type_index, radii, density, diff, relevance);
+    const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
+    abi_check(mg_backward_relevance(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
+                                    type_index.data(), radii.data(), (int)diff.dimension(0),
+                                    reinterpret_cast<const float*>(density.data()),
+                                    reinterpret_cast<const float*>(diff.data()),
+                                    reinterpret_cast<float*>(relevance.data()), nullptr),
+              "GridMaker::backward_relevance");
+  }
+  /// index types, host arrays
+  template <typename Dtype>
+  void backward_relevance(float3 grid_center, const Grid<float, 2, false>& coords,
+                          const Grid<float, 1, false>& type_index, const Grid<float, 1, false>& radii,
+                          const Grid<Dtype, 4, false>& density, const Grid<Dtype, 4, false>& diff,
+                          Grid<Dtype, 1, false>& relevance) const {
+    require_float<Dtype>();
+    check_relevance(coords, type_index, radii, density, diff, relevance);
+    const size_t n = coords.dimension(0);
+    detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_index.data(), n), dr(radii.data(), n);
+    detail::DeviceStaging<float> dd(reinterpret_cast<const float*>(density.data()), density.size());
+    detail::DeviceStaging<float> df(reinterpret_cast<const float*>(diff.data()), diff.size()), drel(n);
+    Grid<float, 2, true> gc(dc.get(), n, 3);
+    Grid<float, 1, true> gt(dt.get(), n), gr(dr.get(), n), grel(drel.get(), n);
+    Grid<float, 4, true> gd(dd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
+    Grid<float, 4, true> gf(df.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
+    backward_relevance(grid_center, gc, gt, gr, gd, gf, grel);
+    drel.download(reinterpret_cast<float*>(relevance.data()));
+  }
+  /// coordinate set (host / device grids)
+  template <typename Dtype>
+  void backward_relevance(float3 grid_center, const CoordinateSet& in, const Grid<Dtype, 4, false>& density,
+                          const Grid<Dtype, 4, false>& diff, Grid<Dtype, 1, false>& relevance) const {
+    if (!in.has_indexed_types()) throw std::invalid_argument("Index types missing from coordinate set in backward relevance");
+    backward_relevance(grid_center, in.coords.cpu(), in.type_index.cpu(), in.radii.cpu(), density, diff, relevance);
+  }
+  template <typename Dtype>
+  void backward_relevance(float3 grid_center, const CoordinateSet& in, const Grid<Dtype, 4, true>& density,
+                          const Grid<Dtype, 4, true>& diff, Grid<Dtype, 1, true>& relevance) const {
+    if (!in.has_indexed_types()) throw std::invalid_argument("Index types missing from coordinate set in backward relevance");
+    backward_relevance(grid_center, in.coords.gpu(), in.type_index.gpu(), in.radii.gpu(), density, diff, relevance);
+  }
+
+  // ---- gradients of the backward pass (grid_maker.h:447-545 of the reference) --------------
+  /// vector types, device arrays; the three outputs are overwritten
+  template <typename Dtype>
+  void backward_gradients(float3 grid_center, const Grid<float, 2, true>& coords,
+                          const Grid<float, 2, true>& type_vectors, const Grid<float, 1, true>& radii,
+                          const Grid<Dtype, 4, true>& diff, const Grid<Dtype, 2, true>& atom_gradients,
+                          const Grid<Dtype, 2, true>& type_gradients, Grid<Dtype, 4, true>& diffdiff,
+                          Grid<Dtype, 2, true>& atom_diffdiff, Grid<Dtype, 2, true>& type_diffdiff) const {
+    require_float<Dtype>();
+    check_backward_gradients(coords, type_vectors, radii, diff, atom_gradients, type_gradients, diffdiff,
+                             atom_diffdiff, type_diffdiff);
+    const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
+    abi_check(mg_backward_gradients(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
+                                    type_vectors.data(), radii.data(), (int)diff.dimension(0),
+                                    reinterpret_cast<const float*>(diff.data()),
+                                    reinterpret_cast<const float*>(atom_gradients.data()),
+                                    reinterpret_cast<const float*>(type_gradients.data()),
+                                    reinterpret_cast<float*>(diffdiff.data()),
+                                    reinterpret_cast<float*>(atom_diffdiff.data()),
+                                    reinterpret_cast<float*>(type_diffdiff.data()), nullptr),
+              "GridMaker::backward_gradients");
+  }
+  /// vector types, host arrays
+  template <typename Dtype>
+  void backward_gradients(float3 grid_center, const Grid<float, 2, false>& coords,
+                          const Grid<float, 2, false>& type_vectors, const Grid<float, 1, false>& radii,
+                          const Grid<Dtype, 4, false>& diff, const Grid<Dtype, 2, false>& atom_gradients,
+                          const Grid<Dtype, 2, false>& type_gradients, Grid<Dtype, 4, false>& diffdiff,
+                          Grid<Dtype, 2, false>& atom_diffdiff, Grid<Dtype, 2, false>& type_diffdiff) const {
+    require_float<Dtype>();
+    check_backward_gradients(coords, type_vectors, radii, diff, atom_gradients, type_gradients, diffdiff,
+                             atom_diffdiff, type_diffdiff);
+    const size_t n = coords.dimension(0), T = type_vectors.dimension(1);
+    detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_vectors.data(), n * T), dr(radii.data(), radii.size());
+    detail::DeviceStaging<float> dd(reinterpret_cast<const float*>(diff.data()), diff.size());
+    detail::DeviceStaging<float> dag(reinterpret_cast<const float*>(atom_gradients.data()), n * 3);
+    detail::DeviceStaging<float> dtg(reinterpret_cast<const float*>(type_gradients.data()), n * T);
+    detail::DeviceStaging<float> odd(diff.size()), oad(n * 3), otd(n * T);
+    Grid<float, 2, true> gc(dc.get(), n, 3), gt(dt.get(), n, T), gag(dag.get(), n, 3), gtg(dtg.get(), n, T);
+    Grid<float, 2, true> goad(oad.get(), n, 3), gotd(otd.get(), n, T);
+    Grid<float, 1, true> gr(dr.get(), radii.size());
+    Grid<float, 4, true> gd(dd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
+    Grid<float, 4, true> godd(odd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
+    backward_gradients(grid_center, gc, gt, gr, gd, gag, gtg, godd, goad, gotd);
+    odd.download(reinterpret_cast<float*>(diffdiff.data()));
+    oad.download(reinterpret_cast<float*>(atom_diffdiff.data()));
+    otd.download(reinterpret_cast<float*>(type_diffdiff.data()));
+  }
+  /// coordinate set with vector types (host / device grids)
+  template <typename Dtype>
+  void backward_gradients(float3 grid_center, const CoordinateSet& in, const Grid<Dtype, 4, false>& diff,
+                          const Grid<Dtype, 2, false>& atom_gradients, const Grid<Dtype, 2, false>& type_gradients,
+                          Grid<Dtype, 4, false>& diffdiff, Grid<Dtype, 2, false>& atom_diffdiff,
+                          Grid<Dtype, 2, false>& type_diffdiff) const {
+    if (!in.has_vector_types()) throw std::invalid_argument("Vector types missing from coordinate set");
+    backward_gradients(grid_center, in.coords.cpu(), in.type_vector.cpu(), in.radii.cpu(), diff, atom_gradients,
+                       type_gradients, diffdiff, atom_diffdiff, type_diffdiff);
+  }
+  template <typename Dtype>
+  void backward_gradients(float3 grid_center, const CoordinateSet& in, const Grid<Dtype, 4, true>& diff,
+                          const Grid<Dtype, 2, true>& atom_gradients, const Grid<Dtype, 2, true>& type_gradients,
+                          Grid<Dtype, 4, true>& diffdiff, Grid<Dtype, 2, true>& atom_diffdiff,
+                          Grid<Dtype, 2, true>& type_diffdiff) const {
+    if (!in.has_vector_types()) throw std::invalid_argument("Vector types missing from coordinate set");
+    backward_gradients(grid_center, in.coords.gpu(), in.type_vector.gpu(), in.radii.gpu(), diff, atom_gradients,
+                       type_gradients, diffdiff, atom_diffdiff, type_diffdiff);
+  }
+
  private:
+  template <typename Dtype, bool isCUDA>
+  void check_relevance(const Grid<float, 2, isCUDA>& coords, const Grid<float, 1, isCUDA>& type_index,
+                       const Grid<float, 1, isCUDA>& radii, const Grid<Dtype, 4, isCUDA>& density,
+                       const Grid<Dtype, 4, isCUDA>& diff, const Grid<Dtype, 1, isCUDA>& relevance) const {
+    const unsigned n = coords.dimension(0);
+    if (n != type_index.size()) throw std::invalid_argument("Type dimension doesn't equal number of coordinates.");
+    if (n != relevance.size()) throw std::invalid_argument("Relevance dimension doesn't equal number of coordinates");
+    if (n != radii.size()) throw std::invalid_argument("Radii dimension doesn't equal number of coordinates");
+    if (coords.dimension(1) != 3) throw std::invalid_argument("Coordinates and radius wrong secondary dimension");
+    for (unsigned i = 0; i <= 3; ++i)
+      if (density.dimension(i) != diff.dimension(i) || (i > 0 && diff.dimension(i) != p.dim))
+        throw std::invalid_argument("density and diff do not have the grid's dimensions");
+  }
+  template <typename Dtype, bool isCUDA>
+  void check_backward_gradients(const Grid<float, 2, isCUDA>& coords, const Grid<float, 2, isCUDA>& type_vector,
+                                const Grid<float, 1, isCUDA>& radii, const Grid<Dtype, 4, isCUDA>& diff,
+                                const Grid<Dtype, 2, isCUDA>& atom_gradients,
+                                const Grid<Dtype, 2, isCUDA>& type_gradients,
+                                const Grid<Dtype, 4, isCUDA>& diffdiff,
+                                const Grid<Dtype, 2, isCUDA>& atom_diffdiff,
+                                const Grid<Dtype, 2, isCUDA>& type_diffdiff) const {
+    check_backward_vector(coords, type_vector, radii, diff, atom_gradients, type_gradients);
+    const unsigned n = coords.dimension(0), ntypes = type_vector.dimension(1);
+    if (n != atom_diffdiff.dimension(0)) throw std::invalid_argument("Atom gradient gradients dimension doesn't equal number of coordinates");
+    if (n != type_diffdiff.dimension(0)) throw std::invalid_argument("Type gradient gradients dimension doesn't equal number of coordinates");
+    if (type_diffdiff.dimension(1) != ntypes) throw std::invalid_argument("Type gradient dimension has wrong number of types");
+    if (p.binary) throw std::invalid_argument("Binary densities not supported");
+    for (unsigned i = 0; i <= 3; ++i)
+      if (diffdiff.dimension(i) != diff.dimension(i))
+        throw std::invalid_argument("diffdiff does not have the dimensions of diff");
+  }
+
   template <typename Dtype, int N>
   void forward_host_batch(const Grid<float, 2, false>& centers, const Grid<float, 3, false>& coords,
                           const Grid<float, N, false>& types, const Grid<float, 2, false>& radii,

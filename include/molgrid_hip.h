@@ -136,6 +136,31 @@ int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
                        const float* diff, float* atom_gradients, float* type_gradients,
                        void* stream);
 
+/* GridMaker::backward_relevance; replaces set_atom_relevance and its launcher
+ * (src/grid_maker.cu:922-992), values of src/grid_maker.cpp:392-432, 680-704.
+ *   density, diff [nbatch, ntypes, dim, dim, dim] -> relevance [n] (overwritten; ignored atoms
+ *   get zero).  Index types only. */
+int mg_backward_relevance(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_index, const float* radii, int ntypes,
+                          const float* density, const float* diff, float* relevance,
+                          void* stream);
+
+/* GridMaker::backward_gradients; replaces set_atom_type_grad_grad and its launcher
+ * (src/grid_maker.cu:652-803), values of src/grid_maker.cpp:529-661.  Vector types, not binary.
+ *   in:  diff [nbatch, ntypes, dim^3], atom_gradients [n,3], type_gradients [n,ntypes]
+ *   out: diffdiff [nbatch, ntypes, dim^3], atom_diffdiff [n,3], type_diffdiff [n,ntypes] (zero);
+ *        all three are overwritten.  diffdiff is summed with float atomics: the order of the
+ *        additions, hence the last bits, can differ from run to run (as in the reference). */
+int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_vector, const float* radii, int ntypes,
+                          const float* diff, const float* atom_gradients,
+                          const float* type_gradients, float* diffdiff, float* atom_diffdiff,
+                          float* type_diffdiff, void* stream);
+
 /* GridInterpolater::forward; replaces gpu_set_outgrid and its per-channel
  * launch loop (src/grid_interpolater.cu:106-166), values of
  * src/grid_interpolater.cpp:16-48.  One launch for all examples and channels.

@@ -1,6 +1,6 @@
 """ctypes binding of the C ABI declared in ``include/molgrid_hip.h``.
 
-The shared library must already be built (``python -m libmolgrid_amd.build``);
+The shared library must already be built (``python libmolgrid_amd/build.py``);
 importing this module fails loudly when it is missing -- there is no fallback.
 """
 import ctypes
@@ -18,7 +18,7 @@ MG_ERR_NULL_POINTER = -4
 EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_vector", "mg_backward_index",
-    "mg_backward_vector", "mg_interpolate",
+    "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate",
 )
 
 
@@ -50,7 +50,7 @@ _f = ctypes.c_float
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            "%s is missing: build it with `python -m libmolgrid_amd.build` "
+            "%s is missing: build it with `python libmolgrid_amd/build.py` "
             "(the gridding kernels have no CPU fallback)" % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH)
     gm = ctypes.POINTER(mg_gridmaker)
@@ -67,6 +67,10 @@ def _load():
     lib.mg_backward_index.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp, _vp]
     lib.mg_backward_vector.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,
                                        _vp, _vp]
+    lib.mg_backward_relevance.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,
+                                          _vp, _vp]
+    lib.mg_backward_gradients.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,
+                                          _vp, _vp, _vp, _vp, _vp]
     lib.mg_interpolate.argtypes = [_f, _f, _f, _f, _i, _i, _vp, _f3, _vp, _vp, _f4, _vp, _f3,
                                    _vp, _f3, _vp, _f3, _vp, _vp]
     for name in EXPORTED_SYMBOLS:

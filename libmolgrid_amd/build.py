@@ -1,6 +1,7 @@
 """Compile the HIP kernels and the C ABI into ``libmolgrid_hip.so`` (gfx950 only).
 
-Run as ``python -m libmolgrid_amd.build``.  hipcc cross-compiles without a GPU.
+Run as ``python libmolgrid_amd/build.py`` (by path: importing the package needs the library
+this script creates).  hipcc cross-compiles without a GPU.
 """
 import os
 import re
@@ -14,7 +15,7 @@ LIB_NAME = "libmolgrid_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
 SOURCES = ["capi.hip", "transform.hip", "forward_index.hip", "forward_vector.hip",
-           "backward.hip", "interpolate.hip"]
+           "backward.hip", "second_order.hip", "interpolate.hip"]
 
 # Packed FP32 instructions are kept out of the generated code.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

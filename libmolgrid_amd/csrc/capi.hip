@@ -232,6 +232,53 @@ int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
                                          g->radii_type_indexed != 0, (hipStream_t)stream));
 }
 
+int mg_backward_relevance(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_index, const float* radii, int ntypes,
+                          const float* density, const float* diff, float* relevance,
+                          void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (coords == nullptr || type_index == nullptr || radii == nullptr || density == nullptr ||
+      diff == nullptr || relevance == nullptr)
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_backward_relevance(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
+                                            vec3(grid_centers, grid_center_host), coords,
+                                            type_index, radii, density, diff, relevance,
+                                            g->binary != 0, (hipStream_t)stream));
+}
+
+int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_vector, const float* radii, int ntypes,
+                          const float* diff, const float* atom_gradients,
+                          const float* type_gradients, float* diffdiff, float* atom_diffdiff,
+                          float* type_diffdiff, void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  // src/grid_maker.cpp:559
+  if (g->binary) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || ntypes == 0) return MG_OK;
+  if (diffdiff == nullptr) return MG_ERR_NULL_POINTER;
+  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
+  if (has_atoms && (coords == nullptr || type_vector == nullptr || radii == nullptr ||
+                    diff == nullptr || atom_gradients == nullptr || type_gradients == nullptr ||
+                    atom_diffdiff == nullptr || type_diffdiff == nullptr))
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_backward_gradients(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
+                                            vec3(grid_centers, grid_center_host), coords,
+                                            type_vector, radii, diff, atom_gradients,
+                                            type_gradients, diffdiff, atom_diffdiff,
+                                            type_diffdiff, g->radii_type_indexed != 0,
+                                            (hipStream_t)stream));
+}
+
 int mg_interpolate(float in_resolution, float in_dimension, float out_resolution,
                    float out_dimension, int nbatch, int channels, const float* in_centers,
                    const float in_center_host[3], const float* in, const float* quats,

@@ -54,6 +54,20 @@ hipError_t launch_backward_vector(const GridArg& g, const BatchArg& batch, int n
                                   float* atom_gradients, float* type_gradients, bool binary,
                                   bool radii_type_indexed, hipStream_t stream);
 
+hipError_t launch_backward_relevance(const GridArg& g, const BatchArg& batch, int nbatch,
+                                     int launch_atoms, const Vec3Arg& centers, const float* coords,
+                                     const float* type_index, const float* radii,
+                                     const float* density, const float* diff, float* relevance,
+                                     bool binary, hipStream_t stream);
+
+hipError_t launch_backward_gradients(const GridArg& g, const BatchArg& batch, int nbatch,
+                                     int launch_atoms, const Vec3Arg& centers,
+                                     const float* coords, const float* type_vector,
+                                     const float* radii, const float* diff,
+                                     const float* atom_gradients, const float* type_gradients,
+                                     float* diffdiff, float* atom_diffdiff, float* type_diffdiff,
+                                     bool radii_type_indexed, hipStream_t stream);
+
 hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_centers,
                               const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
                               const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,

@@ -787,6 +787,109 @@ class GridMaker(object):
         a_ag.finish()
         a_tg.finish()
 
+    def backward_relevance(self, *args):
+        """backward_relevance(center, coordinate_set, density, diff, relevance)
+        backward_relevance(center, coords, type_index, radii, density, diff, relevance)
+
+        include/libmolgrid/grid_maker.h:558-618; values of src/grid_maker.cpp:392-432, 680-704."""
+        if len(args) == 5 and isinstance(args[1], CoordinateSet):
+            center, cs, density, diff, relevance = args
+            if not cs.has_indexed_types():
+                raise ValueError("Index types missing from coordinate set in backward relevance")
+            return self.backward_relevance(center, cs.coords, cs.type_index, cs.radii, density,
+                                           diff, relevance)
+        if len(args) != 7:
+            raise TypeError("backward_relevance expects 5 or 7 arguments")
+        center, coords, types, radii, density, diff, relevance = args
+        c = _to_float3(center)
+        a_coords = _Arg(coords, "coords", 2)
+        a_types = _Arg(types, "type_index", 1)
+        a_radii = _Arg(radii, "radii", 1)
+        a_dens = _Arg(density, "density", 4)
+        a_diff = _Arg(diff, "diff", 4)
+        a_rel = _Arg(relevance, "relevance", 1, out=True)
+        n = a_coords.shape[0]
+        # src/grid_maker.cu:975-978
+        if n != a_types.shape[0]:
+            raise ValueError("Type dimension doesn't equal number of coordinates.")
+        if n != a_rel.shape[0]:
+            raise ValueError("Relevance dimension doesn't equal number of coordinates")
+        if n != a_radii.shape[0]:
+            raise ValueError("Radii dimension doesn't equal number of coordinates")
+        if a_coords.shape[1] != 3:
+            raise ValueError("Coordinates and radius wrong secondary dimension")
+        dim = int(self._p.dim)
+        if a_dens.shape != a_diff.shape or tuple(a_diff.shape[1:]) != (dim, dim, dim):
+            raise ValueError("density and diff must both be (ntypes, %d, %d, %d)" % (dim, dim, dim))
+        code = _lib.mg_backward_relevance(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr,
+                                          a_types.ptr, a_radii.ptr, a_diff.shape[0], a_dens.ptr,
+                                          a_diff.ptr, a_rel.ptr, _stream())
+        _capi.check(code, "GridMaker.backward_relevance")
+        a_rel.finish()
+
+    def backward_gradients(self, *args):
+        """backward_gradients(center, coords, type_vectors, radii, diff, atom_gradients,
+                              type_gradients, diffdiff, atom_diffdiff, type_diffdiff)
+        backward_gradients(center, coordinate_set, diff, atom_gradients, type_gradients,
+                           diffdiff, atom_diffdiff, type_diffdiff)
+
+        Gradients of the backward pass (include/libmolgrid/grid_maker.h:447-545, values of
+        src/grid_maker.cpp:529-661): given gradients with respect to the atom and type gradients,
+        fills the gradient with respect to diff, to the coordinates and to the types (zero)."""
+        if len(args) == 8 and isinstance(args[1], CoordinateSet):
+            cs = args[1]
+            if not cs.has_vector_types():
+                raise ValueError("Vector types missing from coordinate set")
+            return self.backward_gradients(args[0], cs.coords, cs.type_vector, cs.radii, *args[2:])
+        if len(args) != 10:
+            raise TypeError("backward_gradients expects 8 or 10 arguments")
+        center, coords, types, radii, diff, agrad, tgrad, diffdiff, add, tdd = args
+        c = _to_float3(center)
+        a_coords = _Arg(coords, "coords", 2)
+        a_types = _Arg(types, "type_vectors", 2)
+        a_radii = _Arg(radii, "radii", 1)
+        a_diff = _Arg(diff, "diff", 4)
+        a_ag = _Arg(agrad, "atom_gradients", 2)
+        a_tg = _Arg(tgrad, "type_gradients", 2)
+        a_dd = _Arg(diffdiff, "diffdiff", 4, out=True)
+        a_add = _Arg(add, "atom_diffdiff", 2, out=True)
+        a_tdd = _Arg(tdd, "type_diffdiff", 2, out=True)
+        n, T = a_coords.shape[0], a_types.shape[1]
+        dim = int(self._p.dim)
+        # src/grid_maker.cpp:541-559
+        if n != a_types.shape[0]:
+            raise ValueError("Type dimension doesn't equal number of coordinates.")
+        if T != a_diff.shape[0]:
+            raise ValueError("Channels in diff doesn't equal number of types")
+        if n != a_ag.shape[0]:
+            raise ValueError("Atom gradient dimension doesn't equal number of coordinates")
+        if n != a_tg.shape[0]:
+            raise ValueError("Type gradient dimension doesn't equal number of coordinates")
+        if n != a_add.shape[0]:
+            raise ValueError("Atom gradient gradients dimension doesn't equal number of coordinates")
+        if n != a_tdd.shape[0]:
+            raise ValueError("Type gradient gradients dimension doesn't equal number of coordinates")
+        if a_tg.shape[1] != T or a_tdd.shape[1] != T:
+            raise ValueError("Type gradient dimension has wrong number of types")
+        if a_coords.shape[1] != 3 or a_ag.shape[1] != 3 or a_add.shape[1] != 3:
+            raise ValueError("Need x,y,z,r for coord_radius")
+        if self._p.radii_type_indexed:
+            if T != a_radii.shape[0]:
+                raise ValueError("Radii dimension doesn't equal number of types")
+        elif n != a_radii.shape[0]:
+            raise ValueError("Radii dimension doesn't equal number of coordinates")
+        if self._p.binary:
+            raise ValueError("Binary densities not supported")
+        if tuple(a_diff.shape[1:]) != (dim, dim, dim) or a_dd.shape != a_diff.shape:
+            raise ValueError("diff and diffdiff must both be (ntypes, %d, %d, %d)" % (dim, dim, dim))
+        code = _lib.mg_backward_gradients(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr,
+                                          a_types.ptr, a_radii.ptr, T, a_diff.ptr, a_ag.ptr,
+                                          a_tg.ptr, a_dd.ptr, a_add.ptr, a_tdd.ptr, _stream())
+        _capi.check(code, "GridMaker.backward_gradients")
+        a_dd.finish()
+        a_add.finish()
+        a_tdd.finish()
+
     def _backward_padded(self, centers, coords, types, radii, diff, agrad, tgrad=None):
         """Padded batch (B leading): coords (B,N,3), types (B,N) or (B,N,T), radii (B,N),
         diff (B,T,D,D,D) -> gradients shaped like coords / types.  One launch for the batch.

@@ -3,7 +3,8 @@ python/torch_bindings.py:44-163 (``Coords2GridFunction``, ``BatchedCoords2GridFu
 ``Grid2CoordsGradientFunction``, ``Coords2Grid``).
 
 A batch is gridded (and back-propagated) with ONE kernel launch instead of the reference's Python
-loop over examples.  Second-order gradients (``backward_gradients``) are not available.
+loop over examples.  ``Coords2GridFunction`` supports a second backward pass through
+``GridMaker.backward_gradients``, like the reference; the batched function does not.
 """
 import torch
 
@@ -15,15 +16,25 @@ class Grid2CoordsGradientFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, gmaker, center, coords, types, radii, grid_gradient):
+        grid_gradient = grid_gradient.contiguous()
+        ctx.save_for_backward(coords, types, radii, grid_gradient)
+        ctx.gmaker, ctx.center = gmaker, center
         grad_coords = torch.empty_like(coords)
         grad_types = torch.empty_like(types)
-        gmaker.backward(center, coords, types, radii, grid_gradient.contiguous(), grad_coords,
-                        grad_types)
+        gmaker.backward(center, coords, types, radii, grid_gradient, grad_coords, grad_types)
         return grad_coords, grad_types
 
     @staticmethod
     def backward(ctx, grad_coords, grad_types):
-        raise NotImplementedError("second-order gradients of the gridding are not implemented")
+        """Second-order pass (python/torch_bindings.py:59-72)."""
+        coords, types, radii, grid_gradient = ctx.saved_tensors
+        ddcoords = torch.empty_like(coords)
+        ddtypes = torch.empty_like(types)
+        ddG = torch.empty_like(grid_gradient)
+        ctx.gmaker.backward_gradients(ctx.center, coords, types, radii, grid_gradient,
+                                      grad_coords.contiguous(), grad_types.contiguous(), ddG,
+                                      ddcoords, ddtypes)
+        return None, None, ddcoords, ddtypes, None, ddG
 
 
 class Coords2GridFunction(torch.autograd.Function):

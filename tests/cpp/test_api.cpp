@@ -196,6 +196,39 @@ static void gpu_tests() {
   CHECK(eg(2, 16, 12, 12) > 0.99f);   // ligand atom at (1,0,0) lands in channel 2
   CHECK(throws<std::out_of_range>([&] { MGrid4f wrong(2, 25, 25, 25); g1.forward(ex, Transform(), wrong.gpu()); }));
 
+  // relevance: test/test_gridmaker.cpp:313-337
+  {
+    GridMaker gr(0.1, 6.0);
+    CoordinateSet cs(std::vector<float3>{make_float3(0, 0, 0)}, std::vector<int>{0}, std::vector<float>{2.0f}, 1);
+    const unsigned d = gr.get_grid_dims().x;
+    MGrid4f rdiff(1, d, d, d), rdens(1, d, d, d);
+    rdiff(0, 31, 30, 30) = 10.0f;
+    rdens(0, 31, 30, 30) = 1.0f;
+    MGrid1f cpurel(1), gpurel(1);
+    gr.backward_relevance(make_float3(0, 0, 0), cs, rdens.cpu(), rdiff.cpu(), cpurel.cpu());
+    gr.backward_relevance(make_float3(0, 0, 0), cs, rdens.gpu(), rdiff.gpu(), gpurel.gpu());
+    gpurel.tocpu();
+    CHECK_NEAR(cpurel(0), gpurel(0), 1e-5);
+    CHECK(cpurel(0) > 1.0f && cpurel(0) < 10.0f);
+  }
+  // second-order pass: zero upstream gradients give zero everywhere; binary is rejected
+  {
+    GridMaker g2(0.5, 6.0);
+    CoordinateSet cs(std::vector<float3>{make_float3(0.2f, 0, 0)}, std::vector<std::vector<float> >{{1.0f, 0.5f}},
+                     std::vector<float>{1.5f});
+    MGrid4f d4(2, 13, 13, 13), dd4(2, 13, 13, 13);
+    for (size_t i = 0; i < d4.size(); ++i) d4.cpu().data()[i] = 1.0f;
+    MGrid2f ag(1, 3), tg(1, 2), add(1, 3), tdd(1, 2);
+    tg(0, 0) = 1.0f;
+    g2.backward_gradients(make_float3(0, 0, 0), cs, d4.gpu(), ag.gpu(), tg.gpu(), dd4.gpu(), add.gpu(), tdd.gpu());
+    dd4.tocpu(); add.tocpu(); tdd.tocpu();
+    CHECK(tdd(0, 0) == 0 && tdd(0, 1) == 0);
+    CHECK(dd4(0, 6, 6, 6) > 0.9f);      // d(type gradient)/d(diff) is the density itself
+    CHECK(dd4(1, 6, 6, 6) == 0);
+    GridMaker gb(0.5, 6.0, true);
+    CHECK(throws<std::invalid_argument>([&] { gb.backward_gradients(make_float3(0, 0, 0), cs, d4.gpu(), ag.gpu(), tg.gpu(), dd4.gpu(), add.gpu(), tdd.gpu()); }));
+  }
+
   // batch of examples: one packed upload, two launches; equals the per-example calls bit for bit
   Example ex2;
   ex2.sets.push_back(CoordinateSet(p1, std::vector<int>{1}, std::vector<float>{2.0f}, 2));
