@@ -1,9 +1,9 @@
 // Trilinear resampling of a batch of 4-D grids through an inverse rigid transform
 // (GridInterpolater::forward, src/grid_interpolater.cpp:16-48).
 //
-// Main kernel (interpolate_tiled_kernel): one workgroup owns an 8x8x8 tile of output voxels.  The
-// tile maps to a rotated cube in the input grid; the workgroup finds that cube's bounding window
-// (at most 17^3 voxels), stages the window of one channel at a time into LDS with row-coalesced
+// Main kernel (interpolate_tiled_kernel): one workgroup owns an 8x8x16 tile of output voxels (16
+// along z, so that its stores are whole 64-byte lines).  The tile maps to a rotated box in the
+// input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), stages the window of one channel at a time into LDS with row-coalesced
 // loads (zero outside the input grid, so the taps need no bounds tests), and every thread reads
 // its eight taps from LDS.  The source position, tap offsets and weights are computed once per
 // output voxel and reused for every channel; while a channel is being interpolated the next
@@ -60,34 +60,37 @@ __device__ __forceinline__ float lerp3(float p000, float p001, float p010, float
 }
 
 // ---------------------------------------------------------------------------------------------
-constexpr int kTileT = 8;                      // output tile side
-constexpr int kTileThreads = 512;              // one output voxel per thread
-constexpr int kWin = 17;                       // largest staged window side
-constexpr int kWinZ = 18;                      // z stride of the window in LDS (even: 8-byte pairs)
+constexpr int kTileX = 8, kTileY = 8, kTileZ = 16;   // output tile; 16 voxels of z = one 64-byte line
+constexpr int kTileThreads = 512;              // two output voxels (x and x + 4) per thread
+constexpr int kVox = kTileX * kTileY * kTileZ / kTileThreads;
+constexpr int kWin = 21;                       // largest staged window side
+constexpr int kWinZ = 22;                      // z stride of the window in LDS (even: 8-byte pairs)
 constexpr int kWinSize = kWin * kWin * kWinZ;  // floats per buffer
-constexpr int kStagePer = (kWin * kWin * kWin + kTileThreads - 1) / kTileThreads;  // 10
+constexpr int kStagePer = (kWin * kWin * kWin + kTileThreads - 1) / kTileThreads;  // 19
+// longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
+constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
 
 __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
-    InterpArg p, int nbatch, int tiles_per_side, Vec3Arg in_centers, const float* __restrict__ in,
-    Vec4Arg quats, Vec3Arg rot_centers, Vec3Arg translations, Vec3Arg out_centers,
-    float* __restrict__ out) {
-  __shared__ float s_win[2][kWinSize];
+    InterpArg p, int nbatch, int tiles_x, int tiles_z, Vec3Arg in_centers,
+    const float* __restrict__ in, Vec4Arg quats, Vec3Arg rot_centers, Vec3Arg translations,
+    Vec3Arg out_centers, float* __restrict__ out) {
+  extern __shared__ __align__(16) float s_win[];   // two buffers of kWinSize floats, one spare slot
   __shared__ float s_lo[3], s_hi[3];
 
   // workgroup -> (example, tile): consecutive workgroups are dealt round-robin to the 8 XCDs, so
   // example b is pinned to XCD b % 8 and its tiles run there in z-fastest order
-  const int tiles = tiles_per_side * tiles_per_side * tiles_per_side;
+  const int tiles = tiles_x * tiles_x * tiles_z;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int b = (slot / tiles) * 8 + xcd;
   if (b >= nbatch) return;
   const int tile = slot % tiles;
-  const int tz = tile % tiles_per_side, ty = (tile / tiles_per_side) % tiles_per_side;
-  const int tx = tile / (tiles_per_side * tiles_per_side);
+  const int tz = tile % tiles_z, ty = (tile / tiles_z) % tiles_x;
+  const int tx = tile / (tiles_z * tiles_x);
 
   const int od = p.out_dim, id = p.in_dim;
   const int tid = threadIdx.x;
-  const int i = tx * kTileT + (tid >> 6), j = ty * kTileT + ((tid >> 3) & 7), k = tz * kTileT + (tid & 7);
-  const bool live = i < od && j < od && k < od;
+  // 16 consecutive lanes run along z: one store instruction writes whole 64-byte lines
+  const int i0 = tx * kTileX + (tid >> 7), j = ty * kTileY + ((tid >> 4) & 7), k = tz * kTileZ + (tid & 15);
 
   const float3 ic = load3(in_centers, b), oc = load3(out_centers, b);
   const float3 c = load3(rot_centers, b), t = load3(translations, b);
@@ -96,9 +99,9 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   // ---- window of the tile: bounding box of the images of its eight corners -----------------
   if (tid < 8) {
-    const int ci = min(tx * kTileT + ((tid >> 2) & 1) * (kTileT - 1), od - 1);
-    const int cj = min(ty * kTileT + ((tid >> 1) & 1) * (kTileT - 1), od - 1);
-    const int ck = min(tz * kTileT + (tid & 1) * (kTileT - 1), od - 1);
+    const int ci = min(tx * kTileX + ((tid >> 2) & 1) * (kTileX - 1), od - 1);
+    const int cj = min(ty * kTileY + ((tid >> 1) & 1) * (kTileY - 1), od - 1);
+    const int ck = min(tz * kTileZ + (tid & 1) * (kTileZ - 1), od - 1);
     const SourcePoint s = source_point(p, ic, oc, c, t, qinv, qinvinv, ci, cj, ck);
     float lo[3] = {s.gx, s.gy, s.gz}, hi[3] = {s.gx, s.gy, s.gz};
     // min / max over the 8 corner lanes
@@ -128,65 +131,107 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     wn[d] = (int)chi - (int)clo + 1;
   }
 
-  // ---- this thread's taps and weights (channel independent) --------------------------------
-  const SourcePoint s = source_point(p, ic, oc, c, t, qinv, qinvinv, min(i, od - 1), min(j, od - 1),
-                                     min(k, od - 1));
-  const float fx = floorf(s.gx), fy = floorf(s.gy), fz = floorf(s.gz);
-  const float xd = s.gx - fx, yd = s.gy - fy, zd = s.gz - fz;
-  // window-relative tap position, clamped into the window (a clamped tap is outside the input
-  // grid on that side and its neighbours there are zero as well)
-  const int wx = min(max((int)fminf(fmaxf(fx, -4.f), (float)id + 4.f) - wlo[0], 0), wn[0] - 2);
-  const int wy = min(max((int)fminf(fmaxf(fy, -4.f), (float)id + 4.f) - wlo[1], 0), wn[1] - 2);
-  const int wz = min(max((int)fminf(fmaxf(fz, -4.f), (float)id + 4.f) - wlo[2], 0), wn[2] - 2);
-  const int tap = (wx * kWin + wy) * kWinZ + wz;
+  // ---- this thread's taps and corner weights (channel independent) ---------------------------
+  int tap[kVox];
+  float cw[kVox][8];   // weight of tap (x, y, z) at index 4x + 2y + z
+  bool live[kVox];
+#pragma unroll
+  for (int v = 0; v < kVox; ++v) {
+    const int i = i0 + v * (kTileX / kVox);
+    live[v] = i < od && j < od && k < od;
+    const SourcePoint s = source_point(p, ic, oc, c, t, qinv, qinvinv, min(i, od - 1),
+                                       min(j, od - 1), min(k, od - 1));
+    const float fx = floorf(s.gx), fy = floorf(s.gy), fz = floorf(s.gz);
+    // fractional parts; an integral coordinate gives weight 0 to the upper tap
+    const float xd = s.gx - fx, yd = s.gy - fy, zd = s.gz - fz;
+    const float x0 = 1.f - xd, y0 = 1.f - yd, z0 = 1.f - zd;
+    cw[v][0] = x0 * y0 * z0; cw[v][1] = x0 * y0 * zd; cw[v][2] = x0 * yd * z0; cw[v][3] = x0 * yd * zd;
+    cw[v][4] = xd * y0 * z0; cw[v][5] = xd * y0 * zd; cw[v][6] = xd * yd * z0; cw[v][7] = xd * yd * zd;
+    // window-relative tap position, clamped into the window (a clamped tap is outside the input
+    // grid on that side and its neighbours there are zero as well)
+    const int wx = min(max((int)fminf(fmaxf(fx, -4.f), (float)id + 4.f) - wlo[0], 0), wn[0] - 2);
+    const int wy = min(max((int)fminf(fmaxf(fy, -4.f), (float)id + 4.f) - wlo[1], 0), wn[1] - 2);
+    const int wz = min(max((int)fminf(fmaxf(fz, -4.f), (float)id + 4.f) - wlo[2], 0), wn[2] - 2);
+    tap[v] = (wx * kWin + wy) * kWinZ + wz;
+  }
 
   // ---- staging plan of this thread: up to kStagePer window elements per channel ---------------
+  // Window positions outside the input grid hold zero for every channel: both buffers are cleared
+  // once and such positions (and the unused tail of the plan) are steered to a spare LDS slot and
+  // to element 0 of the channel, so that the per-channel loop is load + write without tests.
   const int wcount = wn[0] * wn[1] * wn[2];
   const int plane = wn[1] * wn[2];
-  int st_src[kStagePer];   // offset inside one input channel, or -1 for zero padding / unused
-  int st_dst[kStagePer];   // offset inside the LDS window, or -1 when unused
+  const int rounds = (wcount + kTileThreads - 1) / kTileThreads;   // uniform: rounds in use
+  const float inv_plane = 1.0f / (float)plane, inv_row = 1.0f / (float)wn[2];
+  int st_src[kStagePer];   // offset inside one input channel
+  int st_dst[kStagePer];   // offset inside the LDS window
 #pragma unroll
   for (int e = 0; e < kStagePer; ++e) {
     const int n = tid + e * kTileThreads;
-    st_dst[e] = -1;
-    st_src[e] = -1;
-    if (n < wcount) {
-      const int ex = n / plane, r = n - ex * plane, ey = r / wn[2], ez = r - ey * wn[2];
-      st_dst[e] = (ex * kWin + ey) * kWinZ + ez;
+    st_dst[e] = 2 * kWinSize;   // the spare slot
+    st_src[e] = 0;
+    if (e < rounds && n < wcount) {
+      // n = (ex * wn[1] + ey) * wn[2] + ez; quotients by float reciprocal, corrected by one step
+      int ex = (int)((float)n * inv_plane);
+      ex -= (ex * plane > n) ? 1 : 0;
+      ex += ((ex + 1) * plane <= n) ? 1 : 0;
+      const int r = n - ex * plane;
+      int ey = (int)((float)r * inv_row);
+      ey -= (ey * wn[2] > r) ? 1 : 0;
+      ey += ((ey + 1) * wn[2] <= r) ? 1 : 0;
+      const int ez = r - ey * wn[2];
       const int gx = wlo[0] + ex, gy = wlo[1] + ey, gz = wlo[2] + ez;
-      if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id)
+      if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id) {
+        st_dst[e] = (ex * kWin + ey) * kWinZ + ez;
         st_src[e] = (gx * id + gy) * id + gz;
+      }
     }
   }
+  {
+    float4* z4 = reinterpret_cast<float4*>(s_win);
+    for (int n = tid; n < 2 * kWinSize / 4; n += kTileThreads) z4[n] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  __syncthreads();
 
   const size_t in_chan = (size_t)id * id * id;
   const size_t out_points = (size_t)od * od * od;
   const float* src = in + (size_t)b * p.channels * in_chan;
-  float* dst = out + (size_t)b * p.channels * out_points + ((size_t)i * od + j) * od + k;
+  float* dst = out + (size_t)b * p.channels * out_points + ((size_t)i0 * od + j) * od + k;
+  const size_t vox_step = (size_t)(kTileX / kVox) * od * od;
 
   float staged[kStagePer];
   auto fetch = [&](const float* chan) {
 #pragma unroll
-    for (int e = 0; e < kStagePer; ++e) staged[e] = st_src[e] >= 0 ? chan[st_src[e]] : 0.f;
+    for (int e = 0; e < kStagePer; ++e)
+      if (e < rounds) staged[e] = chan[st_src[e]];
   };
   auto deposit = [&](float* win) {
 #pragma unroll
     for (int e = 0; e < kStagePer; ++e)
-      if (st_dst[e] >= 0) win[st_dst[e]] = staged[e];
+      if (e < rounds) win[st_dst[e]] = staged[e];
   };
 
   fetch(src);
-  deposit(s_win[0]);
+  deposit(s_win);
   __syncthreads();
   for (int ch = 0; ch < p.channels; ++ch) {
     const bool more = ch + 1 < p.channels;
     if (more) fetch(src + (size_t)(ch + 1) * in_chan);   // in flight during the interpolation
-    const float* w = s_win[ch & 1] + tap;
-    const float val = lerp3(w[0], w[1], w[kWinZ], w[kWinZ + 1], w[kWin * kWinZ],
-                            w[kWin * kWinZ + 1], w[kWin * kWinZ + kWinZ],
-                            w[kWin * kWinZ + kWinZ + 1], xd, yd, zd);
-    if (live) dst[(size_t)ch * out_points] = val;
-    if (more) deposit(s_win[(ch + 1) & 1]);
+    const float* buf = s_win + (ch & 1) * kWinSize;
+#pragma unroll
+    for (int v = 0; v < kVox; ++v) {
+      const float* w = buf + tap[v];
+      float val = w[0] * cw[v][0];
+      val = fmaf(w[1], cw[v][1], val);
+      val = fmaf(w[kWinZ], cw[v][2], val);
+      val = fmaf(w[kWinZ + 1], cw[v][3], val);
+      val = fmaf(w[kWin * kWinZ], cw[v][4], val);
+      val = fmaf(w[kWin * kWinZ + 1], cw[v][5], val);
+      val = fmaf(w[kWin * kWinZ + kWinZ], cw[v][6], val);
+      val = fmaf(w[kWin * kWinZ + kWinZ + 1], cw[v][7], val);
+      if (live[v]) dst[(size_t)ch * out_points + v * vox_step] = val;
+    }
+    if (more) deposit(s_win + ((ch + 1) & 1) * kWinSize);
     __syncthreads();
   }
 }
@@ -256,15 +301,20 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
                               const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
                               const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,
                               hipStream_t stream) {
-  // A tile of 8 output voxels per side spans 7 * sqrt(3) * (out_res / in_res) input voxels at
-  // most; with the two extra taps and the rounding slack it must fit the 17-voxel window.
-  const float span = 7.0f * 1.7320508f * (p.out_resolution / p.in_resolution);
-  if (span + 4.0f <= (float)kWin) {
-    const int tiles_per_side = (p.out_dim + kTileT - 1) / kTileT;
-    const int tiles = tiles_per_side * tiles_per_side * tiles_per_side;
+  // The image of an 8 x 8 x 16 output tile spans at most kTileDiagonal * (out_res / in_res) input
+  // voxels along an axis; with the two extra taps and the rounding slack it must fit the window.
+  const float span = kTileDiagonal * (p.out_resolution / p.in_resolution);
+  if (span + 3.0f <= (float)kWin) {
+    const int tiles_x = (p.out_dim + kTileX - 1) / kTileX;
+    const int tiles_z = (p.out_dim + kTileZ - 1) / kTileZ;
+    const int tiles = tiles_x * tiles_x * tiles_z;
     const int groups = (nbatch + 7) / 8;
-    hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), 0,
-                       stream, p, nbatch, tiles_per_side, in_centers, in, quats, rot_centers,
+    const size_t lds = (2 * (size_t)kWinSize + 4) * sizeof(float);   // two buffers and a spare slot
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(interpolate_tiled_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), lds,
+                       stream, p, nbatch, tiles_x, tiles_z, in_centers, in, quats, rot_centers,
                        translations, out_centers, out);
     return hipGetLastError();
   }
