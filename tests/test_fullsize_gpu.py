@@ -1,0 +1,95 @@
+"""The benchmark workload at its full size (batch 50, 28x48^3, 121,231 atoms) through the C ABI:
+every example of the forward pass against the oracle, the gradients of a few examples against the
+oracle, and properties that need no oracle (a batch equals its single launches, reordering atoms
+leaves the binary grid unchanged, the backward pass is linear in the upstream gradient)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import synth
+from test_backward_gpu import check_grads, noise_bound
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mg():
+    import libmolgrid_amd
+    return libmolgrid_amd
+
+
+@pytest.fixture(scope="module")
+def workload():
+    c = synth.config1(nbatch=50)
+    c["moved"] = oracle.transform_forward_batch(c["offsets"], c["quats"], c["centers"],
+                                                c["translations"], c["coords"])
+    return c
+
+
+def test_forward_every_example(mg, workload):
+    c = workload
+    B = len(c["offsets"]) - 1
+    threads = min(oracle.max_threads(), 16)
+    gm = mg.GridMaker(0.5, 23.5)
+    moved, types, radii = dev(c["moved"]), dev(c["types"]), dev(c["radii"])
+    out = torch.full((B,) + gm.grid_dimensions(28), -1.0, device="cuda")
+    gm.forward_batch(c["offsets"], c["centers"], moved, types, radii, out)
+    og = oracle.GridMaker(0.5, 23.5)
+    off = c["offsets"]
+    for b0 in range(0, B, 10):       # ten examples at a time keeps the host copies small
+        ref = og.forward_batch(off[b0:b0 + 11] - off[b0], c["centers"][b0:b0 + 10],
+                               c["moved"][off[b0]:off[b0 + 10]], c["types"][off[b0]:off[b0 + 10]],
+                               c["radii"][off[b0]:off[b0 + 10]], 28, nthreads=threads)
+        got = out[b0:b0 + 10].cpu().numpy()
+        for k in range(ref.shape[0]):
+            assert_close(got[k], ref[k], what="example %d" % (b0 + k))
+    # a batch is its single launches, bit for bit
+    for b in (0, 17, 49):
+        s = slice(off[b], off[b + 1])
+        one = torch.empty(gm.grid_dimensions(28), device="cuda")
+        gm.forward(tuple(c["centers"][b]), moved[s], types[s], radii[s], one)
+        assert torch.equal(one, out[b])
+
+
+def test_binary_grid_ignores_atom_order(mg, workload):
+    c = workload
+    B = len(c["offsets"]) - 1
+    gm = mg.GridMaker(0.5, 23.5, True)
+    out = torch.empty((B,) + gm.grid_dimensions(28), device="cuda")
+    gm.forward_batch(c["offsets"], c["centers"], dev(c["moved"]), dev(c["types"]), dev(c["radii"]),
+                     out)
+    rng = np.random.default_rng(4)
+    perm = np.concatenate([c["offsets"][b] + rng.permutation(c["offsets"][b + 1] - c["offsets"][b])
+                           for b in range(B)])
+    out2 = torch.empty_like(out)
+    gm.forward_batch(c["offsets"], c["centers"], dev(c["moved"][perm]), dev(c["types"][perm]),
+                     dev(c["radii"][perm]), out2)
+    assert torch.equal(out, out2)
+    vals = torch.unique(out)
+    assert vals.tolist() == [0.0, 1.0]
+
+
+def test_backward_full_batch(mg, workload):
+    c = workload
+    B = len(c["offsets"]) - 1
+    off = c["offsets"]
+    gm = mg.GridMaker(0.5, 23.5)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    diff = torch.randn((B,) + gm.grid_dimensions(28), device="cuda", generator=gen)
+    moved, types, radii = dev(c["moved"]), dev(c["types"]), dev(c["radii"])
+    grads = torch.empty((off[-1], 3), device="cuda")
+    gm.backward_batch(off, c["centers"], moved, types, radii, diff, grads)
+    got = grads.cpu().numpy()
+    og = oracle.GridMaker(0.5, 23.5)
+    for b in (0, 23, 49):
+        s = slice(off[b], off[b + 1])
+        d = diff[b].cpu().numpy()
+        args = (c["centers"][b], c["moved"][s], c["types"][s], c["radii"][s], d)
+        check_grads(got[s], og.backward(*args), og.backward(*args, f64=True), noise_bound(og, *args),
+                    "example %d" % b)
+    # linear in the upstream gradient: a factor of two is exact in floating point
+    grads2 = torch.empty_like(grads)
+    gm.backward_batch(off, c["centers"], moved, types, radii, diff * 2, grads2)
+    assert torch.equal(grads2, grads * 2)
