@@ -9,6 +9,7 @@ from ._capi import LIB_PATH, lib as _lib  # noqa: F401  (fails loudly if the .so
 from .gridding import (AtomBatch, CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
                        float3, set_random_seed, transform_batch)
 
+from .grids import *  # noqa: F401,F403,E402  (Grid1f .. Grid8dCUDA, MGrid1f .. MGrid8d, tonumpy)
 from .torch_bindings import (BatchedCoords2GridFunction, Coords2Grid, Coords2GridFunction,  # noqa: F401,E402
                              Grid2CoordsGradientFunction)
 

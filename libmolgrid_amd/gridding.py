@@ -11,12 +11,14 @@ Arrays may be ROCm torch tensors (used in place, on torch's current stream) or
 host arrays (numpy / CPU tensors): host arrays are staged through device memory
 and the kernels still do the work -- there is no CPU implementation here.
 """
+import functools
 import math
 
 import numpy as np
 import torch
 
 from . import _capi
+from . import grids as _grids
 
 _lib = _capi.lib
 
@@ -50,6 +52,7 @@ class float3(object):
 def _to_float3(v):
     if isinstance(v, float3):
         return v
+    v = _unwrap(v)
     if isinstance(v, torch.Tensor):
         v = v.detach().cpu().tolist()
     v = tuple(v)
@@ -166,6 +169,22 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def _unwrap(x):
+    """Grid views and managed grids (grids.py) stand for their tensor; a managed grid for the side
+    its values currently live on (python/bindings_grids.cpp:140-165)."""
+    if isinstance(x, (_grids.GridBase, _grids.ManagedGridBase)):
+        return _grids._tensor_of(x)
+    return x
+
+
+def _accepts_grids(fn):
+    """Lets a public entry point take Grid / MGrid objects wherever it takes an array."""
+    @functools.wraps(fn)
+    def wrapper(*args, **kw):
+        return fn(*[_unwrap(a) for a in args], **{k: _unwrap(v) for k, v in kw.items()})
+    return wrapper
+
+
 class _Arg(object):
     """A user array made visible to the device.
 
@@ -176,6 +195,7 @@ class _Arg(object):
     """
 
     def __init__(self, x, name, ndim, out=False):
+        x = _unwrap(x)
         self.name = name
         self.out = out
         self.host = None
@@ -222,6 +242,7 @@ class _Arg(object):
 
 
 def _same_memory(a, b):
+    a, b = _unwrap(a), _unwrap(b)
     try:
         pa = a.data_ptr() if isinstance(a, torch.Tensor) else a.ctypes.data
         pb = b.data_ptr() if isinstance(b, torch.Tensor) else b.ctypes.data
@@ -231,11 +252,13 @@ def _same_memory(a, b):
 
 
 def _is_host(x):
+    x = _unwrap(x)
     return not (isinstance(x, torch.Tensor) and x.is_cuda)
 
 
 def _small_device(values, width):
     """B x width float32 parameter rows on the device (None -> None)."""
+    values = _unwrap(values)
     if values is None:
         return None
     if isinstance(values, torch.Tensor) and values.is_cuda:
@@ -383,15 +406,18 @@ class Transform(object):
         _capi.check(code, what)
         a_out.finish()
 
+    @_accepts_grids
     def forward(self, src, dst, dotranslate=True):
         """dst = Q.rotate(src - center) + center (+ translate).  In place is fine."""
         self._apply(_lib.mg_transform_forward, "Transform.forward", src, dst, dotranslate)
 
+    @_accepts_grids
     def backward(self, src, dst, dotranslate=True):
         """Inverse: un-translate, then rotate by the inverse about center."""
         self._apply(_lib.mg_transform_backward, "Transform.backward", src, dst, dotranslate)
 
 
+@_accepts_grids
 def transform_batch(offsets, quats, centers, translations, src, dst, dotranslate=True,
                     inverse=False):
     """Apply one rigid transform per example to a packed (ragged) batch of atoms.
@@ -425,7 +451,11 @@ class CoordinateSet(object):
     molecule file needs a chemistry toolkit and is outside the gridding path.
     """
 
+    @_accepts_grids
     def __init__(self, coords, types, radii, max_type=None):
+        # the set owns copies of its arrays (src/coordinateset.cpp:124-160), on the side given
+        coords, types, radii = [x.detach().clone() if isinstance(x, torch.Tensor)
+                                else np.array(x, copy=True) for x in (coords, types, radii)]
         self.coords = coords
         self.radii = radii
         tshape = tuple(types.shape)
@@ -583,6 +613,7 @@ class GridMaker(object):
                                  % (int(np.floor(t).max()), ntypes))
 
     # -- forward ------------------------------------------------------------
+    @_accepts_grids
     def forward(self, *args, **kw):
         """forward(center, coordinate_set, grid)
         forward(center, coords, types, radii, grid)          one example
@@ -657,6 +688,7 @@ class GridMaker(object):
         _capi.check(code, "GridMaker.forward")
         a_out.finish()
 
+    @_accepts_grids
     def forward_batch(self, offsets, centers, coords, types, radii, grid):
         """Ragged batch in one launch: example b owns atoms offsets[b]:offsets[b+1] of the
         packed arrays; centers (B,3); grid (B,T,D,D,D).  With type-indexed radii,
@@ -697,6 +729,7 @@ class GridMaker(object):
         a_out.finish()
 
     # -- backward -----------------------------------------------------------
+    @_accepts_grids
     def backward(self, *args):
         """backward(center, coordinate_set, diff, atom_gradients[, type_gradients])
         backward(center, coords, type_index, radii, diff, atom_gradients)
@@ -787,6 +820,7 @@ class GridMaker(object):
         a_ag.finish()
         a_tg.finish()
 
+    @_accepts_grids
     def backward_relevance(self, *args):
         """backward_relevance(center, coordinate_set, density, diff, relevance)
         backward_relevance(center, coords, type_index, radii, density, diff, relevance)
@@ -827,6 +861,7 @@ class GridMaker(object):
         _capi.check(code, "GridMaker.backward_relevance")
         a_rel.finish()
 
+    @_accepts_grids
     def backward_gradients(self, *args):
         """backward_gradients(center, coords, type_vectors, radii, diff, atom_gradients,
                               type_gradients, diffdiff, atom_diffdiff, type_diffdiff)
@@ -950,6 +985,7 @@ class GridMaker(object):
         a_ag.finish()
         a_tg.finish()
 
+    @_accepts_grids
     def backward_batch(self, offsets, centers, coords, types, radii, diff, atom_gradients,
                        type_gradients=None):
         """Ragged batch in one launch; diff is (B,T,D,D,D); gradients are packed like the
@@ -1069,6 +1105,7 @@ class GridInterpolater(object):
             raise ValueError("Output grid wrong dimension. Should be %d along all axes but is "
                              "%d,%d,%d" % ((self.out_dim,) + tuple(out_shape[1:])))
 
+    @_accepts_grids
     def forward(self, *args, **kw):
         """forward(in, transform, out)
         forward(in_center, in, transform, out_center, out)
@@ -1100,6 +1137,7 @@ class GridInterpolater(object):
         _capi.check(code, "GridInterpolater.forward")
         a_out.finish()
 
+    @_accepts_grids
     def forward_batch(self, src, quats, rot_centers, translations, dst, in_centers=None,
                       out_centers=None):
         """One launch for a batch: src (B,K,Din,Din,Din) -> dst (B,K,Dout,Dout,Dout) with one
