@@ -62,10 +62,40 @@ __device__ __forceinline__ float point_density(const GridArg& g, float dx, float
   return density<BINARY, false>(g, dx, dy, dz, BINARY ? ar2 : inv_ar2, 0.f, frm2, grm2);
 }
 
+// a * b with 0 * anything = 0 (also infinities and NaNs)
+__device__ __forceinline__ float mul_zero_wins(float a, float b) {
+  float r;
+  asm("v_mul_legacy_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// Voxel range [lo, lo + n) along one axis whose centres lie within `reach` of `coord` (n <= 0:
+// none).  Tighter than the reference's index box (src/grid_maker.cu:66-79), which adds a voxel
+// beyond the reach on either side; such voxels contribute nothing to a gradient.  The slack keeps
+// every voxel that rounding could put on the inner side of the cut-off: whether it counts is
+// decided by the distance test of the voxel itself.
+__device__ __forceinline__ void reach_range(float origin, float coord, float reach, float inv_res,
+                                            int dim, int& lo, int& n) {
+  constexpr float kSlack = 1e-3f;
+  const float first = fmaxf(ceilf((coord - reach - origin) * inv_res - kSlack), 0.f);
+  const float last = fminf(floorf((coord + reach - origin) * inv_res + kSlack), (float)(dim - 1));
+  lo = (int)first;
+  n = (int)last - lo + 1;
+}
+
+// Atom gradients for index types.  One wave per atom.  The (y, z) columns of the atom's box that
+// come within reach of the atom are compacted into a wave-private list (a circle's worth of
+// columns instead of the square's), each lane takes one column of the list and marches along x;
+// the offset in x of plane i is computed by lane i beforehand and read back as a scalar.  Per
+// voxel the lane adds scale*dx to its x partial and scale to a running sum: dy and dz are fixed
+// along the march, so the y and z partials are that sum times dy and dz.
 __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_index, const float* __restrict__ radii,
     const float* __restrict__ diff, float* __restrict__ atom_gradients) {
+  // column list of each wave: (j << 16 | k) offsets inside the atom's box; a chunk of candidates
+  // adds at most kWave entries to fewer than kWave pending ones
+  __shared__ int s_cols[kBwdWaves][2 * kWave];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so is the atom
   const int b = blockIdx.y;
@@ -77,10 +107,14 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
   const float oz = center.z - g.half_dimension;
   const int dim = g.dim;
   const size_t chan_stride = (size_t)dim * dim * dim;
+  const unsigned plane_stride = (unsigned)(dim * dim);
   const float* diff_b = diff + (size_t)b * g.ntypes * chan_stride;
+  const float inv_res = 1.0f / g.resolution;
+  volatile int* cols = s_cols[wave];
+  constexpr int kPlanes = 8;    // planes of a column in flight together
 
   for (int a = begin + blockIdx.x * kBwdWaves + wave; a < end; a += gridDim.x * kBwdWaves) {
-    float gx = 0.f, gy = 0.f, gz = 0.f;
+    float gx = 0.f, gy = 0.f, gz = 0.f, gauss = 0.f;
     const float tf = roundf(type_index[a]);  // backward rounds, forward floors
     if (tf >= 0.f && tf < (float)g.ntypes) {
       const float ax = coords[3 * a], ay = coords[3 * a + 1], az = coords[3 * a + 2];
@@ -91,26 +125,98 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
         densityrad = radius * g.radius_scale * g.frm;
         ar = radius * g.radius_scale;
       }
-      const GradConsts gc = grad_consts(g, ar);
-      int lo0, hi0, lo1, hi1, lo2, hi2;
-      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
-      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
-      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
-      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
+      // scale = -(1/dist) d(density)/d(dist) (density_grad_dist, src/grid_maker.cu:881-898), in
+      // terms of dist^2 and divided by 4/ar^2 (the partial sums are multiplied by it at the end):
+      // Gaussian core  exp(-2 dist^2/ar^2) = exp2(exp_k dist^2);  quadratic tail
+      // -(D/ar^2 + E/(ar dist)) ar^2/4 = quad_b/dist + quad_a, which falls to zero at the cut-off
+      // and is negative beyond, so clamping at zero applies the cut-off.
+      const float inv_ar = 1.0f / ar;
+      const float inv_ar2 = inv_ar * inv_ar;
+      const float exp_k = inv_ar2 * kNeg2Log2e;
+      gauss = 4.0f * inv_ar2;
+      const float quad_a = -0.25f * g.D;
+      const float quad_b = -0.25f * g.E * ar;
+      const float core2 = g.grm * g.grm * ar * ar;
+      const float reach2 = densityrad * densityrad;
+      int lo0, lo1, lo2, ni, nj, nk;
+      reach_range(ox, ax, densityrad, inv_res, dim, lo0, ni);
+      reach_range(oy, ay, densityrad, inv_res, dim, lo1, nj);
+      reach_range(oz, az, densityrad, inv_res, dim, lo2, nk);
       if (ni > 0 && nj > 0 && nk > 0) {
         const float* chan = diff_b + (size_t)(int)tf * chan_stride;
-        sweep_channel(g, chan, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
-                      [&](float dx, float dy, float dz, float dist2, float gv, bool) {
-                        const float sc = grad_scale(gc, dist2, gv);
-                        gx = fmaf(dx, sc, gx);
-                        gy = fmaf(dy, sc, gy);
-                        gz = fmaf(dz, sc, gz);
-                      });
+        const int ncols = nj * nk;
+        const float inv_nk = __builtin_amdgcn_rcpf((float)nk);
+        for (int i0 = 0; i0 < ni; i0 += kWave) {
+          const int planes = min(kWave, ni - i0);
+          const float dx_mine = grid_coord(ox, lo0 + i0 + lane, g.resolution) - ax;
+          const int dx_lane = __float_as_int(dx_mine);
+          // planes that lie beyond the Gaussian core as a whole skip its exponential
+          const unsigned long long tail_planes = __ballot(dx_mine * dx_mine > core2);
+          const float* first_plane = chan + (size_t)(unsigned)(lo0 + i0) * plane_stride;
+
+          // one pass: lanes below `count` take the columns cols[0 .. count)
+          auto march = [&](int count) {
+            const bool live = lane < count;
+            const int packed = cols[live ? lane : 0];
+            const int j = packed >> 16, k = packed & 0xffff;
+            const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+            const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+            const float dyz2 = live ? dy * dy + dz * dz : INFINITY;
+            const unsigned lane_off = (unsigned)((lo1 + j) * dim + lo2 + k);
+            float sum = 0.f;
+            for (int i = 0; i < planes; i += kPlanes) {
+              const float* p = first_plane + (size_t)(unsigned)i * plane_stride;
+              float gv[kPlanes];
+#pragma unroll
+              for (int u = 0; u < kPlanes; ++u)
+                if (i + u < planes) gv[u] = (p + (size_t)u * plane_stride)[lane_off];
+#pragma unroll
+              for (int u = 0; u < kPlanes; ++u) {
+                if (i + u < planes) {
+                  const float dx = __int_as_float(__builtin_amdgcn_readlane(dx_lane, i + u));
+                  const float dist2 = fmaf(dx, dx, dyz2);
+                  const float tail =
+                      fmaxf(fmaf(quad_b, __builtin_amdgcn_rsqf(dist2), quad_a), 0.f);
+                  float s = tail;
+                  if (!((tail_planes >> (i + u)) & 1ull)) {
+                    const float core = __builtin_amdgcn_exp2f(dist2 * exp_k);
+                    s = dist2 <= core2 ? core : tail;
+                  }
+                  // 0 * x = 0 for every x: a voxel out of reach adds nothing whatever diff holds
+                  const float sc = mul_zero_wins(s, gv[u]);
+                  gx = fmaf(dx, sc, gx);
+                  sum += sc;
+                }
+              }
+            }
+            gy = fmaf(dy, sum, gy);
+            gz = fmaf(dz, sum, gz);
+          };
+
+          int pending = 0;
+          for (int c0 = 0; c0 < ncols; c0 += kWave) {
+            const int cand = c0 + lane;
+            const int j = (int)(((float)cand + 0.5f) * inv_nk), k = cand - j * nk;
+            const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+            const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+            const bool within = cand < ncols && dy * dy + dz * dz <= reach2;
+            const unsigned long long m = __ballot(within);
+            if (within) cols[pending + __popcll(m & ((1ull << lane) - 1ull))] = (j << 16) | k;
+            pending += __popcll(m);
+            if (pending >= kWave) {
+              march(kWave);
+              pending -= kWave;
+              const int moved = cols[kWave + lane];
+              if (lane < pending) cols[lane] = moved;
+            }
+          }
+          if (pending > 0) march(pending);
+        }
       }
     }
-    gx = wave_sum(gx);
-    gy = wave_sum(gy);
-    gz = wave_sum(gz);
+    gx = wave_sum(gx) * gauss;
+    gy = wave_sum(gy) * gauss;
+    gz = wave_sum(gz) * gauss;
     if (lane == 0) {
       atom_gradients[3 * a] = gx;
       atom_gradients[3 * a + 1] = gy;

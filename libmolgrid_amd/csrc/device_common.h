@@ -46,6 +46,24 @@ __device__ __forceinline__ void example_range(const BatchArg& a, int b, int& beg
   }
 }
 
+// Which example the workgroups of launch slot `slot` (blockIdx.y) work on.  Workgroups start in
+// launch order and the time of one grows with the atoms of its example, so a ragged batch is
+// taken largest example first: the workgroups still running when the launch drains are then the
+// cheapest ones.  Ties keep their order; batches with equal sizes, or with more examples than a
+// wave has lanes, keep the launch order.  Every lane of the wave must call this.
+__device__ __forceinline__ int example_for_slot(const BatchArg& a, int slot, int nbatch, int lane) {
+  if (a.offsets == nullptr || nbatch < 2 || nbatch > kWave) return slot;
+  const int me = lane < nbatch ? lane : nbatch - 1;
+  const int mine = a.offsets[me + 1] - a.offsets[me];
+  int before = 0;   // examples that come before this lane's in (size descending, index) order
+  for (int i = 0; i < nbatch; ++i) {
+    const int other = __builtin_amdgcn_readlane(mine, i);
+    before += (other > mine || (other == mine && i < lane)) ? 1 : 0;
+  }
+  const unsigned long long hit = __ballot(lane < nbatch && before == slot);
+  return hit ? (int)__builtin_ctzll(hit) : slot;
+}
+
 // Scalars every gridding kernel needs (a flattened mg_gridmaker plus derived
 // values computed once on the host).
 struct GridArg {

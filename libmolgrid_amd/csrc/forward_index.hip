@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kColThreads) void splat_column_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
-  const int b = blockIdx.y;
+  const int b = example_for_slot(batch, blockIdx.y, gridDim.y, lane);
   int begin, end;
   example_range(batch, b, begin, end);
   const float3 center = load3(centers, b);
