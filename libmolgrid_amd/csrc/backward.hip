@@ -62,6 +62,8 @@ __device__ __forceinline__ float point_density(const GridArg& g, float dx, float
   return density<BINARY, false>(g, dx, dy, dz, BINARY ? ar2 : inv_ar2, 0.f, frm2, grm2);
 }
 
+constexpr int kRawBufferFlags = 0x00020000;   // untyped 32-bit elements, no swizzle (gfx9 family)
+
 // a * b with 0 * anything = 0 (also infinities and NaNs)
 __device__ __forceinline__ float mul_zero_wins(float a, float b) {
   float r;
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
   const float* diff_b = diff + (size_t)b * g.ntypes * chan_stride;
   const float inv_res = 1.0f / g.resolution;
   volatile int* cols = s_cols[wave];
-  constexpr int kPlanes = 8;    // planes of a column in flight together
+  constexpr int kPlanes = 16;   // planes of a column in flight together
 
   for (int a = begin + blockIdx.x * kBwdWaves + wave; a < end; a += gridDim.x * kBwdWaves) {
     float gx = 0.f, gy = 0.f, gz = 0.f, gauss = 0.f;
@@ -152,7 +154,6 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
           const int dx_lane = __float_as_int(dx_mine);
           // planes that lie beyond the Gaussian core as a whole skip its exponential
           const unsigned long long tail_planes = __ballot(dx_mine * dx_mine > core2);
-          const float* first_plane = chan + (size_t)(unsigned)(lo0 + i0) * plane_stride;
 
           // one pass: lanes below `count` take the columns cols[0 .. count)
           auto march = [&](int count) {
@@ -165,11 +166,21 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
             const unsigned lane_off = (unsigned)((lo1 + j) * dim + lo2 + k);
             float sum = 0.f;
             for (int i = 0; i < planes; i += kPlanes) {
-              const float* p = first_plane + (size_t)(unsigned)i * plane_stride;
+              // buffer loads: the plane's offset is a scalar operand and the column's a 32-bit
+              // vector one, so no address arithmetic is left to the vector unit; slots past the
+              // last plane read the last plane again and are not used
+              const size_t first = (size_t)(unsigned)(lo0 + i0 + i) * plane_stride;
+              const size_t bytes = (chan_stride - first) * sizeof(float);
+              const __amdgpu_buffer_rsrc_t planes_of_chan = __builtin_amdgcn_make_buffer_rsrc(
+                  const_cast<float*>(chan + first), 0,
+                  (int)(bytes < 0xffffffffull ? bytes : 0xffffffffull), kRawBufferFlags);
+              const int last = planes - 1 - i;
               float gv[kPlanes];
 #pragma unroll
               for (int u = 0; u < kPlanes; ++u)
-                if (i + u < planes) gv[u] = (p + (size_t)u * plane_stride)[lane_off];
+                gv[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    planes_of_chan, (int)(lane_off * 4u),
+                    (int)((unsigned)min(u, last) * plane_stride * 4u), 0));
 #pragma unroll
               for (int u = 0; u < kPlanes; ++u) {
                 if (i + u < planes) {
