@@ -135,6 +135,60 @@ def test_ragged_batch_vs_oracle(mg, sparse):
     assert np.array_equal(grads.cpu().numpy(), un_ref)
 
 
+@pytest.mark.parametrize("gm_args", [
+    dict(gaussian_radius_multiple=-1.5),              # truncated Gaussian, no quadratic tail
+    dict(gaussian_radius_multiple=2.0),
+    dict(radius_scale=0.5, gaussian_radius_multiple=3.0),
+    dict(radius_scale=1.7),
+    dict(binary=True),                                # the gradient ignores the binary flag
+])
+def test_unusual_radius_multiples(mg, gm_args):
+    """The tail of the gradient scale is cut off by clamping it at zero, which relies on the tail
+    reaching zero at the final radius for every choice of the multiples (src/grid_maker.cpp:20-36)."""
+    rng = np.random.default_rng(77)
+    natoms, ntypes = 40, 4
+    coords, types, radii = synth.small_index_case(rng, natoms, ntypes, 7.0)
+    og = oracle.GridMaker(0.5, 11.5, **gm_args)
+    diff = rng.standard_normal(og.grid_shape(ntypes)).astype(np.float32)
+    center = (0.3, -0.2, 0.1)
+    ref32 = og.backward(center, coords, types, radii, diff)
+    ref64 = og.backward(center, coords, types, radii, diff, f64=True)
+    mag = noise_bound(og, center, coords, types, radii, diff)
+    gm = mg.GridMaker(0.5, 11.5, **gm_args)
+    grads = torch.full((natoms, 3), 9.0, device="cuda")
+    gm.backward(center, dev(coords), dev(types), dev(radii), dev(diff), grads)
+    check_grads(grads.cpu().numpy(), ref32, ref64, mag, "backward %r" % (gm_args,))
+
+
+def test_values_out_of_reach_are_never_used(mg):
+    """A voxel beyond the final radius is skipped whatever it holds
+    (density_grad_dist returns NaN there and the term is dropped, src/grid_maker.cu:884-915)."""
+    og = oracle.GridMaker(0.5, 11.5)
+    gm = mg.GridMaker(0.5, 11.5)
+    coords = np.asarray([[0.1, 0.2, -0.3], [2.0, -1.0, 0.7]], np.float32)
+    types = np.asarray([0, 0], np.float32)
+    radii = np.asarray([1.5, 1.2], np.float32)
+    rng = np.random.default_rng(5)
+    diff = rng.standard_normal(og.grid_shape(1)).astype(np.float32)
+    ref = og.backward((0, 0, 0), coords, types, radii, diff)
+    # poison every voxel farther than the final radius from both atoms
+    ax = np.arange(24) * 0.5 - 5.75
+    X, Y, Z = np.meshgrid(ax, ax, ax, indexing="ij")
+    far = np.ones(X.shape, bool)
+    for c, r in zip(coords, radii):
+        far &= np.sqrt((X - c[0]) ** 2 + (Y - c[1]) ** 2 + (Z - c[2]) ** 2) > 1.5 * r + 1e-3
+    poisoned = diff.copy()
+    poisoned[0][far] = np.where(rng.random(int(far.sum())) < 0.5, np.inf, np.nan)
+    grads = torch.empty((2, 3), device="cuda")
+    gm.backward((0, 0, 0), dev(coords), dev(types), dev(radii), dev(poisoned), grads)
+    got = grads.cpu().numpy()
+    assert np.isfinite(got).all()
+    clean = torch.empty((2, 3), device="cuda")
+    gm.backward((0, 0, 0), dev(coords), dev(types), dev(radii), dev(diff), clean)
+    assert np.array_equal(got, clean.cpu().numpy())
+    assert_close(got, ref, rtol=1e-4, atol=1e-5, what="poisoned grid vs oracle on the clean one")
+
+
 def test_repeat_runs_are_bit_identical(mg):
     c = synth.config1(nbatch=2)
     gm = mg.GridMaker(0.5, 23.5)
