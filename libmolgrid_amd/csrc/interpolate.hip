@@ -3,20 +3,24 @@
 //
 // Main kernel (interpolate_tiled_kernel): one workgroup owns an 8x8x16 tile of output voxels (16
 // along z, so that its stores are whole 64-byte lines).  The tile maps to a rotated box in the
-// input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), stages the window of one channel at a time into LDS with row-coalesced
-// loads (zero outside the input grid, so the taps need no bounds tests), and every thread reads
-// its eight taps from LDS.  The source position, tap offsets and weights are computed once per
-// output voxel and reused for every channel; while a channel is being interpolated the next
-// channel's window is already in flight (double-buffered LDS, one barrier per channel).
-// Workgroups are numbered so that all tiles of one example run on the same XCD (they share its
-// input through that XCD's L2) and z-neighbouring tiles, which complete each other's cache lines
-// in the output, run back to back.
+// input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), marks the
+// window positions that some tap of the tile reads (about 40 % of the window: the rest of the
+// bounding box is never touched), deals those positions out evenly to its threads, and then stages
+// them one channel at a time into LDS (zero outside the input grid, so the taps need no bounds
+// tests); every thread reads its eight taps from LDS.  The source position, tap offsets and
+// weights are computed once per output voxel and reused for every channel.  Staging runs two
+// channels ahead of the interpolation: two register sets and two LDS buffers, one barrier per
+// channel.  Workgroups are numbered so that all tiles of one example run on the same XCD (they
+// share its input through that XCD's L2) and z-neighbouring tiles, which complete each other's
+// cache lines in the output, run back to back.
 //
 // Fallback kernel (interpolate_gather_kernel): one thread per output voxel gathering its taps
 // straight from global memory; used when a tile's window would not fit (strong down-sampling).
 //
 // The coordinate chain keeps the reference's rounding order; taps outside the input grid read as
 // zero and integral coordinates get weight zero (src/grid_interpolater.cu:17-58).
+#include <cstdlib>
+
 #include "kernels.h"
 
 namespace mg {
@@ -62,20 +66,23 @@ __device__ __forceinline__ float lerp3(float p000, float p001, float p010, float
 // ---------------------------------------------------------------------------------------------
 constexpr int kTileX = 8, kTileY = 8, kTileZ = 16;   // output tile; 16 voxels of z = one 64-byte line
 constexpr int kTileThreads = 512;              // two output voxels (x and x + 4) per thread
+constexpr int kTileWaves = kTileThreads / 64;
 constexpr int kVox = kTileX * kTileY * kTileZ / kTileThreads;
 constexpr int kWin = 21;                       // largest staged window side
 constexpr int kWinZ = 22;                      // z stride of the window in LDS (even: 8-byte pairs)
 constexpr int kWinSize = kWin * kWin * kWinZ;  // floats per buffer
 constexpr int kStagePer = (kWin * kWin * kWin + kTileThreads - 1) / kTileThreads;  // 19
+constexpr int kFewRounds = 6;                  // staged elements per thread and channel (6 x 512 >= 2,800)
 // longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
 constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
 
 __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     InterpArg p, int nbatch, int tiles_x, int tiles_z, Vec3Arg in_centers,
     const float* __restrict__ in, Vec4Arg quats, Vec3Arg rot_centers, Vec3Arg translations,
-    Vec3Arg out_centers, float* __restrict__ out) {
+    Vec3Arg out_centers, float* __restrict__ out, int plain_staging) {
   extern __shared__ __align__(16) float s_win[];   // two buffers of kWinSize floats, one spare slot
   __shared__ float s_lo[3], s_hi[3];
+  __shared__ int s_scan[kStagePer * kTileWaves + 1];
 
   // workgroup -> (example, tile): consecutive workgroups are dealt round-robin to the 8 XCDs, so
   // example b is pinned to XCD b % 8 and its tiles run there in z-fastest order
@@ -155,10 +162,31 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     tap[v] = (wx * kWin + wy) * kWinZ + wz;
   }
 
+  // ---- which window positions any voxel of the tile reads ------------------------------------
+  // The window is the bounding box of a rotated tile, so most of it is never touched.  One byte per
+  // window position (the window's own LDS, before it is first filled): every thread marks its
+  // sixteen taps.
+  {
+    unsigned char* used = reinterpret_cast<unsigned char*>(s_win);
+    unsigned* used4 = reinterpret_cast<unsigned*>(s_win);
+    for (int n = tid; n < (kWinSize + 3) / 4; n += kTileThreads) used4[n] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < kVox; ++v) {
+      if (live[v]) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          used[tap[v] + (c >> 2) * (kWin * kWinZ) + ((c >> 1) & 1) * kWinZ + (c & 1)] = 1;
+      }
+    }
+    __syncthreads();
+  }
+
   // ---- staging plan of this thread: up to kStagePer window elements per channel ---------------
   // Window positions outside the input grid hold zero for every channel: both buffers are cleared
-  // once and such positions (and the unused tail of the plan) are steered to a spare LDS slot and
-  // to element 0 of the channel, so that the per-channel loop is load + write without tests.
+  // once and such positions, the positions no tap reads and the unused tail of the plan are
+  // steered to a spare LDS slot and to element 0 of the channel, so that the per-channel loop is
+  // load + write without tests.
   const int wcount = wn[0] * wn[1] * wn[2];
   const int plane = wn[1] * wn[2];
   const int rounds = (wcount + kTileThreads - 1) / kTileThreads;   // uniform: rounds in use
@@ -181,12 +209,80 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
       ey += ((ey + 1) * wn[2] <= r) ? 1 : 0;
       const int ez = r - ey * wn[2];
       const int gx = wlo[0] + ex, gy = wlo[1] + ey, gz = wlo[2] + ez;
-      if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id) {
-        st_dst[e] = (ex * kWin + ey) * kWinZ + ez;
+      const int cell = (ex * kWin + ey) * kWinZ + ez;
+      if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id &&
+          reinterpret_cast<const unsigned char*>(s_win)[cell] != 0) {
+        st_dst[e] = cell;
         st_src[e] = (gx * id + gy) * id + gz;
       }
     }
   }
+  // ---- the planned elements, compacted: every thread gets an equal share of the ones in use --
+  // Slots are numbered in window order (round, wave, lane), so neighbouring lanes still load
+  // neighbouring addresses.  Counts per (round, wave) go to LDS, wave 0 turns them into offsets,
+  // the (source, destination) pairs are written to a list in the window's LDS and read back
+  // strided by the workgroup size.
+  int* counts = reinterpret_cast<int*>(s_scan);            // [kStagePer][kTileWaves] + total
+  const int lane = tid & 63, wave = tid >> 6;
+  int before[kStagePer];                                   // planned elements of the wave before this lane
+#pragma unroll
+  for (int e = 0; e < kStagePer; ++e) {
+    const unsigned long long m = __ballot(st_dst[e] != 2 * kWinSize);
+    before[e] = __popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) counts[e * kTileWaves + wave] = __popcll(m);
+  }
+  __syncthreads();   // counts complete; every thread has read the marks
+  if (wave == 0) {
+    constexpr int kCounts = kStagePer * kTileWaves;        // 152
+    constexpr int kPerLane = (kCounts + 63) / 64;          // 3
+    int mine[kPerLane], sum = 0;
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) {
+      const int i = lane * kPerLane + q;
+      mine[q] = i < kCounts ? counts[i] : 0;
+      sum += mine[q];
+    }
+    int incl = sum;                                        // inclusive scan over the lanes
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    int run = incl - sum;
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) {
+      const int i = lane * kPerLane + q;
+      if (i < kCounts) counts[i] = run;
+      run += mine[q];
+    }
+    if (lane == 63) counts[kCounts] = incl;
+  }
+  __syncthreads();
+  {
+    int* list = reinterpret_cast<int*>(s_win);             // pairs: source offset, destination
+#pragma unroll
+    for (int e = 0; e < kStagePer; ++e) {
+      if (st_dst[e] != 2 * kWinSize) {
+        const int slot = counts[e * kTileWaves + wave] + before[e];
+        list[2 * slot] = st_src[e];
+        list[2 * slot + 1] = st_dst[e];
+      }
+    }
+  }
+  __syncthreads();
+  const int planned = counts[kStagePer * kTileWaves];
+  const int rounds_used = (planned + kTileThreads - 1) / kTileThreads;   // uniform
+  {
+    const int* list = reinterpret_cast<const int*>(s_win);
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e) {
+      const int slot = tid + e * kTileThreads;
+      const bool mine = slot < planned;
+      st_src[e] = mine ? list[2 * slot] : 0;
+      st_dst[e] = mine ? list[2 * slot + 1] : 2 * kWinSize;
+    }
+  }
+  __syncthreads();   // every thread holds its share: the window can be cleared
   {
     float4* z4 = reinterpret_cast<float4*>(s_win);
     for (int n = tid; n < 2 * kWinSize / 4; n += kTileThreads) z4[n] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -199,25 +295,9 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   float* dst = out + (size_t)b * p.channels * out_points + ((size_t)i0 * od + j) * od + k;
   const size_t vox_step = (size_t)(kTileX / kVox) * od * od;
 
-  float staged[kStagePer];
-  auto fetch = [&](const float* chan) {
-#pragma unroll
-    for (int e = 0; e < kStagePer; ++e)
-      if (e < rounds) staged[e] = chan[st_src[e]];
-  };
-  auto deposit = [&](float* win) {
-#pragma unroll
-    for (int e = 0; e < kStagePer; ++e)
-      if (e < rounds) win[st_dst[e]] = staged[e];
-  };
-
-  fetch(src);
-  deposit(s_win);
-  __syncthreads();
-  for (int ch = 0; ch < p.channels; ++ch) {
-    const bool more = ch + 1 < p.channels;
-    if (more) fetch(src + (size_t)(ch + 1) * in_chan);   // in flight during the interpolation
-    const float* buf = s_win + (ch & 1) * kWinSize;
+  // channel `ch` of the tile from the window buffer that holds it
+  auto interpolate_channel = [&](int ch, int which) {
+    const float* buf = s_win + which * kWinSize;
 #pragma unroll
     for (int v = 0; v < kVox; ++v) {
       const float* w = buf + tap[v];
@@ -231,7 +311,66 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
       val = fmaf(w[kWin * kWinZ + kWinZ + 1], cw[v][7], val);
       if (live[v]) dst[(size_t)ch * out_points + v * vox_step] = val;
     }
-    if (more) deposit(s_win + ((ch + 1) & 1) * kWinSize);
+  };
+  const int C = p.channels;
+
+  if (rounds_used > kFewRounds || plain_staging) {
+    // More planned elements than the register sets below hold.  The launcher sends only resolution
+    // ratios here for which a tile needs at most 2,800 input voxels (the cells that meet the
+    // rotated 7 x 7 x 15 box grown by the taps), so this is a safety net: every thread copies
+    // whole-window elements straight into one buffer, working out the positions as it goes.
+    const float inv_plane_ = 1.0f / (float)plane, inv_row_ = 1.0f / (float)wn[2];
+    for (int ch = 0; ch < C; ++ch) {
+      const float* chan = src + (size_t)ch * in_chan;
+      for (int n = tid; n < wcount; n += kTileThreads) {
+        int ex = (int)((float)n * inv_plane_);
+        ex -= (ex * plane > n) ? 1 : 0;
+        ex += ((ex + 1) * plane <= n) ? 1 : 0;
+        const int r = n - ex * plane;
+        int ey = (int)((float)r * inv_row_);
+        ey -= (ey * wn[2] > r) ? 1 : 0;
+        ey += ((ey + 1) * wn[2] <= r) ? 1 : 0;
+        const int ez = r - ey * wn[2];
+        const int gx = wlo[0] + ex, gy = wlo[1] + ey, gz = wlo[2] + ez;
+        if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id)
+          s_win[(ex * kWin + ey) * kWinZ + ez] = chan[(gx * id + gy) * id + gz];
+      }
+      __syncthreads();
+      interpolate_channel(ch, 0);
+      __syncthreads();
+    }
+    return;
+  }
+
+  // Two register sets, so that the loads of a channel are issued a whole channel before they are
+  // needed: while channel ch is interpolated from one buffer, channel ch + 1 is written to the
+  // other and channel ch + 2 is in flight.
+  float ra[kFewRounds], rb[kFewRounds];
+  auto fetch = [&](float (&r)[kFewRounds], int ch) {
+    const float* chan = src + (size_t)ch * in_chan;
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e)
+      if (e < rounds_used) r[e] = chan[st_src[e]];
+  };
+  auto deposit = [&](const float (&r)[kFewRounds], int ch) {
+    float* win = s_win + (ch & 1) * kWinSize;
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e)
+      if (e < rounds_used) win[st_dst[e]] = r[e];
+  };
+  fetch(ra, 0);
+  deposit(ra, 0);
+  if (C > 1) fetch(ra, 1);
+  __syncthreads();
+  for (int ch = 0; ch < C; ch += 2) {
+    if (ch + 2 < C) fetch(rb, ch + 2);
+    if (ch + 1 < C) deposit(ra, ch + 1);
+    interpolate_channel(ch, 0);
+    __syncthreads();
+    if (ch + 1 >= C) break;
+    if (ch + 3 < C) fetch(ra, ch + 3);
+    if (ch + 2 < C) deposit(rb, ch + 2);
+    interpolate_channel(ch + 1, 1);
     __syncthreads();
   }
 }
@@ -310,12 +449,15 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
     const int tiles = tiles_x * tiles_x * tiles_z;
     const int groups = (nbatch + 7) / 8;
     const size_t lds = (2 * (size_t)kWinSize + 4) * sizeof(float);   // two buffers and a spare slot
+    // test hook: take the plain staging path (otherwise only a safety net) for every tile
+    const char* hook = getenv("MOLGRID_HIP_INTERP_PLAIN_STAGING");
+    const int plain_staging = (hook != nullptr && hook[0] == '1') ? 1 : 0;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(interpolate_tiled_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), lds,
                        stream, p, nbatch, tiles_x, tiles_z, in_centers, in, quats, rot_centers,
-                       translations, out_centers, out);
+                       translations, out_centers, out, plain_staging);
     return hipGetLastError();
   }
   const int out_points = p.out_dim * p.out_dim * p.out_dim;

@@ -69,6 +69,27 @@ def test_batch_config4_shape_vs_oracle(mg):
     assert_close(out.cpu().numpy(), ref, what="config 4")
 
 
+def test_plain_staging_path_gives_the_same_values(mg, monkeypatch):
+    """The kernel's safety net (whole-window staging, taken when a tile would need more input voxels
+    than the pipelined path holds) is not reachable with valid resolutions; the library's test hook
+    forces it, and it must reproduce the pipelined path bit for bit."""
+    rng = np.random.default_rng(9)
+    B, K, D = 2, 5, 48
+    src = dev(rng.standard_normal((B, K, D, D, D)).astype(np.float32))
+    quats = synth.random_quaternions(rng, B)
+    trans = rng.uniform(-1.5, 1.5, (B, 3)).astype(np.float32)
+    zeros = np.zeros((B, 3), np.float32)
+    gi = mg.GridInterpolater(0.5, 23.5, 0.5, 23.5)
+    fast = torch.empty((B, K, D, D, D), device="cuda")
+    gi.forward_batch(src, quats, zeros, trans, fast)
+    monkeypatch.setenv("MOLGRID_HIP_INTERP_PLAIN_STAGING", "1")
+    plain = torch.full((B, K, D, D, D), 7.0, device="cuda")
+    gi.forward_batch(src, quats, zeros, trans, plain)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOLGRID_HIP_INTERP_PLAIN_STAGING")
+    assert torch.equal(fast, plain)
+
+
 def test_argument_errors(mg):
     gi = mg.GridInterpolater(0.5, 6.0, 0.5, 6.0)
     g = torch.zeros((2, 13, 13, 13), device="cuda")
