@@ -6,8 +6,8 @@ C ABI of ``include/molgrid_hip.h``; this package is the Python host side that
 mirrors the reference's ``molgrid`` module for that path.
 """
 from ._capi import LIB_PATH, lib as _lib  # noqa: F401  (fails loudly if the .so is missing)
-from .gridding import (AtomBatch, CoordinateSet, GridInterpolater, GridMaker, Quaternion, Transform,  # noqa: F401
-                       float3, set_random_seed, transform_batch)
+from .gridding import (AtomBatch, CoordinateSet, Example, ExampleVec, GridInterpolater, GridMaker,  # noqa: F401
+                       Quaternion, Transform, float3, set_random_seed, transform_batch)
 
 from .grids import *  # noqa: F401,F403,E402  (Grid1f .. Grid8dCUDA, MGrid1f .. MGrid8d, tonumpy)
 from .torch_bindings import (BatchedCoords2GridFunction, Coords2Grid, Coords2GridFunction,  # noqa: F401,E402

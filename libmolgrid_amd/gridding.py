@@ -444,62 +444,464 @@ def transform_batch(offsets, quats, centers, translations, src, dst, dotranslate
 # --------------------------------------------------------------------------- #
 # CoordinateSet (array constructors only)
 # --------------------------------------------------------------------------- #
+def _managed(x, ndim, cols=None):
+    """Managed float32 grid holding a copy of x (array, tensor or grid), on the side x is on."""
+    x = _unwrap(x)
+    if isinstance(x, torch.Tensor):
+        t = x.detach()
+    else:
+        t = torch.from_numpy(np.ascontiguousarray(np.asarray(x, dtype=np.float32)))
+    if t.dim() != ndim:
+        raise ValueError("expected a %d-dimensional array, got %d dimensions" % (ndim, t.dim()))
+    if cols is not None and t.dim() == 2 and t.shape[1] != cols and t.shape[0] > 0:
+        raise ValueError("expected %d columns, got %d" % (cols, t.shape[1]))
+    m = _grids._mgrid_class(ndim, "f")(*[int(d) for d in t.shape])
+    if t.is_cuda:
+        m.togpu()
+    m.copyFrom(t.to(torch.float32).contiguous())
+    return m
+
+
+def _resized_copy(src, *shape):
+    """Managed grid of the given shape holding the leading elements of src (flat order), on the
+    side src is on (ManagedGrid::resized, include/libmolgrid/managed_grid.h)."""
+    m = _grids._mgrid_class(len(shape), "f")(*shape)
+    if src.ongpu():
+        m.togpu()
+    m.copyFrom(src)
+    return m
+
+
 class CoordinateSet(object):
-    """Atoms of one molecule: coords (N,3), index types (N) or type vectors
-    (N,T), radii (N).  Only the array constructors of
-    include/libmolgrid/coordinateset.h:60-92 exist here; building one from a
-    molecule file needs a chemistry toolkit and is outside the gridding path.
+    """Atoms of one molecule: ``coords`` (N,3), ``type_index`` (N, integers stored as floats) or
+    ``type_vector`` (N,T), ``radii`` (N, or T once the radii are indexed by type), all managed
+    grids that the set owns (include/libmolgrid/coordinateset.h:33-120).
+
+      CoordinateSet()                                   empty
+      CoordinateSet(coords, type_index, radii, max_type)
+      CoordinateSet(coords, type_vector, radii)
+      CoordinateSet(rec, lig, unique_index_types=True)  rec followed by lig
+
+    Building one from a molecule file needs a chemistry toolkit and is outside the gridding path.
     """
 
     @_accepts_grids
-    def __init__(self, coords, types, radii, max_type=None):
-        # the set owns copies of its arrays (src/coordinateset.cpp:124-160), on the side given
-        coords, types, radii = [x.detach().clone() if isinstance(x, torch.Tensor)
-                                else np.array(x, copy=True) for x in (coords, types, radii)]
-        self.coords = coords
-        self.radii = radii
-        tshape = tuple(types.shape)
-        if len(tshape) == 1:
-            if max_type is None:
-                raise ValueError("max_type is required with index types")
-            self.type_index, self.type_vector = types, None
-            self.max_type = int(max_type)
-        elif len(tshape) == 2:
-            self.type_index, self.type_vector = None, types
-            self.max_type = tshape[1]
-        else:
+    def __init__(self, *args, **kw):
+        self.coords = _grids.MGrid2f(0, 3)
+        self.type_index = _grids.MGrid1f(0)
+        self.type_vector = _grids.MGrid2f(0, 0)
+        self.radii = _grids.MGrid1f(0)
+        self.max_type = 0
+        self.src = None
+        if not args and not kw:
+            return
+        if isinstance(args[0], CoordinateSet):
+            names = ("rec", "lig", "unique_index_types")
+            vals = dict(zip(names, args))
+            vals.update(kw)
+            self.mergeInto(vals["rec"], vals["lig"], vals.get("unique_index_types", True))
+            return
+        names = ("coords", "types", "radii", "max_type")
+        vals = dict(zip(names, args))
+        vals.update(kw)
+        coords, types, radii = vals["coords"], vals["types"], vals["radii"]
+        max_type = vals.get("max_type")
+        tdim = len(tuple(types.shape))
+        if tdim not in (1, 2):
             raise ValueError("types must be 1-D (indices) or 2-D (vectors)")
         n = tuple(coords.shape)[0]
-        if tshape[0] != n:
+        if tuple(types.shape)[0] != n:
             raise ValueError("Types and coordinates are of different sizes")
-        if tuple(radii.shape)[0] != n and len(tshape) == 1:
-            raise ValueError("Radii and coordinates are of different sizes")
+        self.coords = _managed(coords, 2, 3)
+        self.radii = _managed(radii, 1)
+        if tdim == 1:
+            # src/coordinateset.cpp:124-128
+            if max_type is None:
+                raise ValueError("max_type is required with index types")
+            if self.radii.size() != n:
+                raise ValueError("Radii and coordinates are of different sizes")
+            self.type_index = _managed(types, 1)
+            self.max_type = int(max_type)
+        else:
+            # src/coordinateset.cpp:161-166
+            self.type_vector = _managed(types, 2)
+            self.max_type = int(tuple(types.shape)[1])
 
+    # -- typing ---------------------------------------------------------------------------
     def has_indexed_types(self):
-        return self.type_index is not None
+        return self.type_index.size() > 0 or self.coords.size() == 0
 
     def has_vector_types(self):
-        return self.type_vector is not None
+        return self.type_vector.size() > 0 or self.coords.size() == 0
 
-    def size(self):
-        return tuple(self.coords.shape)[0]
-
-    def __len__(self):
-        return self.size()
+    def make_vector_types(self, include_dummy_type=False, type_radii=()):
+        """One-hot vectors from the index types, in place; with ``type_radii`` the radii become
+        indexed by type (src/coordinateset.cpp:187-213)."""
+        type_radii = [float(r) for r in type_radii]
+        if type_radii and len(type_radii) != self.max_type:
+            raise ValueError("Type radii size %d does not equal max type %d"
+                             % (len(type_radii), self.max_type))
+        if include_dummy_type:
+            self.max_type += 1
+        idx = self.type_index.tonumpy()
+        n = idx.shape[0]
+        vec = np.zeros((n, self.max_type), np.float32)
+        t = idx.astype(np.int64)
+        ok = (idx >= 0) & (t < self.max_type)
+        vec[np.nonzero(ok)[0], t[ok]] = 1.0
+        on_gpu = self.coords.ongpu()
+        self.type_vector = _grids.MGrid2f(n, self.max_type)
+        self.type_vector.copyFrom(vec)
+        if on_gpu:
+            self.type_vector.togpu()
+        if type_radii:
+            r = np.zeros(self.max_type, np.float32)
+            r[:len(type_radii)] = type_radii
+            self.radii = _grids.MGrid1f(self.max_type)
+            self.radii.copyFrom(r)
 
     def num_types(self):
         return self.max_type
 
+    def set_num_types(self, maxt):
+        self.max_type = int(maxt)
+
+    def sum_types(self, out, zerofirst=True):
+        """out[t] (+)= number of atoms of type t, or the column sums of the type vectors
+        (src/coordinateset.cpp:340-365)."""
+        o = _unwrap(out)
+        if tuple(o.shape) != (self.max_type,):
+            raise ValueError("Type sum output dimension does not match number of types: %d vs %d"
+                             % (tuple(o.shape)[0], self.max_type))
+        if not (self.has_vector_types() and self.type_vector.size() > 0):
+            t = np.round(self.type_index.tonumpy()).astype(np.int64)
+            t = t[t >= 0]
+            if t.size and t.max() >= self.max_type:
+                raise IndexError("Somehow an index type is too large (internal error).")
+            sums = np.bincount(t, minlength=self.max_type).astype(np.float32)
+        else:
+            sums = self.type_vector.tonumpy().sum(axis=0, dtype=np.float32)
+        if isinstance(o, torch.Tensor):
+            add = torch.from_numpy(sums).to(o.device, o.dtype)
+            if zerofirst:
+                o.copy_(add)
+            else:
+                o.add_(add)
+        elif zerofirst:
+            o[...] = sums
+        else:
+            o += sums
+
+    # -- size, centre ---------------------------------------------------------------------
+    def size(self):
+        return self.coords.dimension(0)
+
+    def __len__(self):
+        return self.size()
+
     def center(self):
-        """Mean coordinate (src/coordinateset.cpp:214-229)."""
-        c = self.coords
-        if isinstance(c, torch.Tensor):
-            c = c.detach().cpu().numpy()
-        c = np.asarray(c, dtype=np.float64)
-        if c.shape[0] == 0:
+        """Mean coordinate, summed in float in atom order (src/coordinateset.cpp:214-229)."""
+        n = self.size()
+        if n == 0:
             return float3()
-        m = c.mean(axis=0)
-        return float3(*m)
+        c = self.coords.tonumpy()
+        s = np.cumsum(c, axis=0, dtype=np.float32)[-1]
+        return float3(*(s / np.float32(n)))
+
+    # -- copies ---------------------------------------------------------------------------
+    def clone(self):
+        c = CoordinateSet()
+        c.coords, c.type_index = self.coords.clone(), self.type_index.clone()
+        c.type_vector, c.radii = self.type_vector.clone(), self.radii.clone()
+        c.max_type, c.src = self.max_type, self.src
+        return c
+
+    def togpu(self, copy=True):
+        for g in (self.coords, self.type_index, self.type_vector, self.radii):
+            g.togpu()
+
+    def tocpu(self, copy=True):
+        for g in (self.coords, self.type_index, self.type_vector, self.radii):
+            g.tocpu()
+
+    def copyInto(self, other):
+        c = other.clone()
+        self.coords, self.type_index, self.type_vector = c.coords, c.type_index, c.type_vector
+        self.radii, self.max_type, self.src = c.radii, c.max_type, c.src
+
+    def copyTo(self, coords, types, radii):
+        """Copy into the caller's arrays, truncating what does not fit and leaving what is beyond
+        untouched; type vectors go row by row when the widths differ.  Returns the number of
+        coordinates copied (src/coordinateset.cpp:300-337)."""
+        c, t, r = _unwrap(coords), _unwrap(types), _unwrap(radii)
+        if tuple(c.shape)[1] != 3:
+            raise ValueError("Coordinates have wrong secondary dimension in copyTo")
+        copied = self.coords.copyTo(c)
+        self.radii.copyTo(r)
+        if len(tuple(t.shape)) == 1:
+            self.type_index.copyTo(t)
+        elif self.type_vector.size() > 0 and tuple(t.shape)[1] != self.type_vector.dimension(1):
+            src = _grids._tensor_of(self.type_vector)
+            dst = t if isinstance(t, torch.Tensor) else torch.from_numpy(t)
+            rows = min(dst.shape[0], src.shape[0])
+            cols = min(dst.shape[1], src.shape[1])
+            dst[:rows, :cols].copy_(src[:rows, :cols])
+        else:
+            self.type_vector.copyTo(t)
+        return copied // 3
+
+    def mergeInto(self, rec, lig, unique_index_types=True):
+        """This set becomes rec followed by lig; with unique_index_types the index types of lig
+        are shifted past those of rec (src/coordinateset.cpp:258-298)."""
+        if rec.type_vector.dimension(1) != lig.type_vector.dimension(1):
+            raise ValueError("Type vectors are incompatible sizes")
+        if (rec.has_vector_types() != lig.has_vector_types()) and \
+                (rec.has_indexed_types() != lig.has_indexed_types()):
+            raise ValueError("Incompatible types when combining coodinate sets")
+        if rec.has_indexed_types():
+            max_type = rec.max_type + lig.max_type if unique_index_types \
+                else max(rec.max_type, lig.max_type)
+        else:
+            if rec.max_type != lig.max_type:
+                raise ValueError("Type vectors are incompatible sizes, weirdly")
+            max_type = self.max_type
+        on_gpu = rec.coords.ongpu()
+
+        def joined(a, b, ndim, cols=None):
+            x, y = a.tonumpy(), b.tonumpy()
+            if ndim == 2:
+                x = x.reshape(x.shape[0], cols)
+                y = y.reshape(y.shape[0], cols)
+            m = _managed(np.concatenate([x, y]), ndim)
+            if on_gpu:
+                m.togpu()
+            return m
+
+        nr = rec.type_index.size()
+        coords = joined(rec.coords, lig.coords, 2, 3)
+        tindex = np.concatenate([rec.type_index.tonumpy(), lig.type_index.tonumpy()])
+        if unique_index_types:
+            tindex[nr:] += np.float32(rec.max_type)
+        tvec = joined(rec.type_vector, lig.type_vector, 2, rec.type_vector.dimension(1))
+        radii = joined(rec.radii, lig.radii, 1)
+        self.coords, self.type_vector, self.radii = coords, tvec, radii
+        self.type_index = _managed(tindex, 1)
+        if on_gpu:
+            self.type_index.togpu()
+        self.max_type = max_type
+
+    def __eq__(self, other):
+        if not isinstance(other, CoordinateSet):
+            return NotImplemented
+        return (self.max_type == other.max_type and
+                all(np.array_equal(a.tonumpy(), b.tonumpy()) for a, b in (
+                    (self.coords, other.coords), (self.type_index, other.type_index),
+                    (self.type_vector, other.type_vector), (self.radii, other.radii))))
+
+    __hash__ = None
+
+
+class Example(object):
+    """The coordinate sets (receptor, ligand, ...) and labels of one training example
+    (include/libmolgrid/example.h:29-110)."""
+
+    def __init__(self):
+        self.coord_sets = []
+        self.labels = []
+        self.group = -1
+        self.seqcont = False
+
+    @property
+    def sets(self):
+        return self.coord_sets
+
+    def num_coordinates(self):
+        return sum(c.size() for c in self.coord_sets)
+
+    def num_types(self, unique_index_type=True):
+        if unique_index_type:
+            return sum(c.max_type for c in self.coord_sets)
+        return max([c.max_type for c in self.coord_sets] + [0])
+
+    def has_vector_types(self, start=0):
+        return all(c.has_vector_types() for c in self.coord_sets[start:] if c.size() > 0)
+
+    def has_index_types(self, start=0):
+        return all(c.has_indexed_types() for c in self.coord_sets[start:] if c.size() > 0)
+
+    def togpu(self):
+        for c in self.coord_sets:
+            c.togpu()
+
+    def tocpu(self):
+        for c in self.coord_sets:
+            c.tocpu()
+
+    def _merged_arrays(self, start, unique_index_types, vector):
+        """coords, types, radii of the sets from `start` on as numpy arrays
+        (src/example.cpp:69-100 and 138-195)."""
+        sets = self.coord_sets[start:]
+        if not vector:
+            coords, types, radii, toffset = [], [], [], 0
+            for cs in sets:
+                if cs.size() == 0:
+                    continue
+                if not cs.has_indexed_types():
+                    raise RuntimeError("Coordinate sets do not have compatible index types for merge.")
+                coords.append(cs.coords.tonumpy())
+                types.append(cs.type_index.tonumpy() + np.float32(toffset))
+                radii.append(cs.radii.tonumpy())
+                if unique_index_types:
+                    toffset += cs.max_type
+            if not coords:
+                return (np.zeros((0, 3), np.float32), np.zeros(0, np.float32),
+                        np.zeros(0, np.float32))
+            return np.concatenate(coords), np.concatenate(types), np.concatenate(radii)
+        maxt = 0
+        for i, cs in enumerate(sets):
+            maxt = maxt + cs.max_type if unique_index_types else max(maxt, cs.max_type)
+            if cs.size() == 0:
+                continue
+            if not cs.has_vector_types():
+                raise RuntimeError("Coordinate sets do not have compatible vector types for merge.")
+            if cs.max_type != cs.type_vector.dimension(1):
+                raise RuntimeError("Coordinate set %d does not have consistent max_type/vector "
+                                   "type sizes" % (start + i))
+        coords, types, radii, offset = [], [], [], 0
+        for cs in sets:
+            n = cs.size()
+            tv = cs.type_vector.tonumpy().reshape(n, -1)
+            if offset + tv.shape[1] > maxt and n > 0:
+                raise RuntimeError("Incompatible vector sizes in merge_coordinates")
+            block = np.zeros((n, maxt), np.float32)
+            block[:, offset:offset + tv.shape[1]] = tv
+            coords.append(cs.coords.tonumpy().reshape(n, 3))
+            types.append(block)
+            radii.append(cs.radii.tonumpy())
+            if unique_index_types:
+                offset += cs.max_type
+        if not coords:
+            return (np.zeros((0, 3), np.float32), np.zeros((0, maxt), np.float32),
+                    np.zeros(0, np.float32))
+        return np.concatenate(coords), np.concatenate(types), np.concatenate(radii)
+
+    def merge_coordinates(self, *args, **kw):
+        """merge_coordinates(start=0, unique_index_types=True) -> CoordinateSet
+        merge_coordinates(coord, types, radius, start=0, unique_index_types=True)   fills arrays
+        (src/example.cpp:40-67, 102-136 and 197-228)."""
+        if args and not isinstance(args[0], (int, bool)):
+            names = ("coord", "types", "radius", "start", "unique_index_types")
+            vals = dict(zip(names, args))
+            vals.update(kw)
+            c, t, r = _unwrap(vals["coord"]), _unwrap(vals["types"]), _unwrap(vals["radius"])
+            vector = len(tuple(t.shape)) == 2
+            coords, types, radii = self._merged_arrays(vals.get("start", 0),
+                                                       vals.get("unique_index_types", True), vector)
+            if vector and types.shape[0] == 0:
+                return
+            if tuple(c.shape)[0] != coords.shape[0]:
+                raise ValueError("Coordinates do not have correct dimension: %d != %d"
+                                 % (tuple(c.shape)[0], coords.shape[0]))
+            if tuple(c.shape)[1] != 3:
+                raise ValueError("Coordinates do not have correct second dimension (3): %d"
+                                 % tuple(c.shape)[1])
+            if tuple(t.shape) != types.shape:
+                raise ValueError("Types do not have correct dimension: %r != %r"
+                                 % (tuple(t.shape), types.shape))
+            if tuple(r.shape)[0] != radii.shape[0]:
+                raise ValueError("Radii do not have correct dimension: %d != %d"
+                                 % (tuple(r.shape)[0], radii.shape[0]))
+            for dst, src in ((c, coords), (t, types), (r, radii)):
+                if isinstance(dst, torch.Tensor):
+                    dst.copy_(torch.from_numpy(src))
+                else:
+                    dst[...] = src
+            return
+        names = ("start", "unique_index_types")
+        vals = dict(zip(names, args))
+        vals.update(kw)
+        start, unique = int(vals.get("start", 0)), bool(vals.get("unique_index_types", True))
+        has_vec, has_ind = self.has_vector_types(), self.has_index_types()
+        if not has_ind and not has_vec:
+            raise ValueError("Inconsistent typing schemes in merge_coordinates")
+        if len(self.coord_sets) <= start:
+            return CoordinateSet()
+        if len(self.coord_sets) == start + 1:
+            return self.coord_sets[start].clone()
+        if not has_vec:
+            coords, types, radii = self._merged_arrays(start, unique, False)
+            return CoordinateSet(coords, types, radii, self.num_types(unique))
+        coords, types, radii = self._merged_arrays(start, unique, True)
+        return CoordinateSet(coords, types, radii)
+
+    def sum_types(self, out, unique_types=True):
+        """src/example.cpp:345-368"""
+        o = _unwrap(out)
+        nt = self.num_types(unique_types)
+        if tuple(o.shape) != (nt,):
+            raise ValueError("Size of sum output doesn't match number of types in example: %d vs %d"
+                             % (tuple(o.shape)[0], nt))
+        if not unique_types:
+            o[...] = 0
+            for cs in self.coord_sets:
+                if cs.num_types() == nt:
+                    cs.sum_types(o, False)
+                else:
+                    part = np.zeros(cs.num_types(), np.float32)
+                    cs.sum_types(part)
+                    if isinstance(o, torch.Tensor):
+                        o[:part.shape[0]] += torch.from_numpy(part).to(o.device)
+                    else:
+                        o[:part.shape[0]] += part
+            return
+        offset = 0
+        for cs in self.coord_sets:
+            n = cs.num_types()
+            if n == 0:
+                continue
+            cs.sum_types(o[offset:offset + n])
+            offset += n
+
+
+class ExampleVec(list):
+    """A batch of examples, as ExampleProvider.next_batch returns it (python/bindings.in.cpp)."""
+
+    def extract_labels(self, out):
+        """out[i, :] = labels of example i (src/example.cpp:254-272)."""
+        o = _unwrap(out)
+        if tuple(o.shape)[0] != len(self):
+            raise IndexError("Grid dimension does not match number of examples: %d vs %d"
+                             % (tuple(o.shape)[0], len(self)))
+        if not self:
+            return
+        nlabels = len(self[0].labels)
+        if tuple(o.shape)[1] != nlabels:
+            raise IndexError("Grid dimension does not match number of labels: %d vs %d"
+                             % (nlabels, tuple(o.shape)[1]))
+        if any(len(ex.labels) != nlabels for ex in self):
+            raise RuntimeError("Non-uniform number of labels")
+        vals = np.asarray([ex.labels for ex in self], np.float32).reshape(len(self), nlabels)
+        if isinstance(o, torch.Tensor):
+            o.copy_(torch.from_numpy(vals))
+        else:
+            o[...] = vals
+
+    def extract_label(self, labelpos, out):
+        """out[i] = label `labelpos` of example i (src/example.cpp:278-299)."""
+        o = _unwrap(out)
+        if tuple(o.shape)[0] != len(self):
+            raise IndexError("Grid dimension does not match number of examples")
+        if not self:
+            return
+        if labelpos >= len(self[0].labels):
+            raise IndexError("labelpos invalid: %d >= %d" % (labelpos, len(self[0].labels)))
+        if any(labelpos >= len(ex.labels) for ex in self):
+            raise IndexError("labelpos invalid (nonuniform labels)")
+        vals = np.asarray([ex.labels[labelpos] for ex in self], np.float32)
+        if isinstance(o, torch.Tensor):
+            o.copy_(torch.from_numpy(vals))
+        else:
+            o[...] = vals
 
 
 # --------------------------------------------------------------------------- #
@@ -618,7 +1020,29 @@ class GridMaker(object):
         """forward(center, coordinate_set, grid)
         forward(center, coords, types, radii, grid)          one example
         forward(centers, coords, types, radii, grid)         padded batch (B leading)
+        forward(example, transform, grid)                    grid centred at the rotation centre
+        forward(example, grid, random_translation=0, random_rotation=False, center=None)
+        forward(examples, grid5, random_translation=0, random_rotation=False)
         ``types`` is 1-D per example for index types, 2-D for type vectors."""
+        if args and isinstance(args[0], Example):
+            if len(args) >= 3 and isinstance(args[1], Transform):
+                if kw or len(args) != 3:
+                    raise TypeError("forward(example, transform, grid) expected")
+                return self._forward_example(args[0], args[1], args[2])
+            names = ("grid", "random_translation", "random_rotation", "center")
+            vals = dict(zip(names, args[1:]))
+            vals.update(kw)
+            t = Transform(self._example_center(args[0], vals.get("center")),
+                          vals.get("random_translation", 0.0), vals.get("random_rotation", False))
+            return self._forward_example(args[0], t, vals["grid"])
+        if args and isinstance(args[0], (list, tuple)) and \
+                (len(args[0]) == 0 or isinstance(args[0][0], Example)):
+            names = ("grid", "random_translation", "random_rotation")
+            vals = dict(zip(names, args[1:]))
+            vals.update(kw)
+            return self._forward_examples(args[0], vals["grid"],
+                                          vals.get("random_translation", 0.0),
+                                          vals.get("random_rotation", False))
         if kw:
             raise TypeError("forward takes positional arguments only")
         if len(args) == 3:
@@ -626,8 +1050,6 @@ class GridMaker(object):
             if not isinstance(cs, CoordinateSet):
                 raise TypeError("forward(center, CoordinateSet, grid) expected")
             types = cs.type_vector if cs.has_vector_types() and cs.size() > 0 else cs.type_index
-            if types is None:
-                types = cs.type_vector
             return self.forward(center, cs.coords, types, cs.radii, grid)
         if len(args) != 5:
             raise TypeError("forward expects 3 or 5 arguments")
@@ -654,6 +1076,65 @@ class GridMaker(object):
                   a_out.shape[0], a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward")
         a_out.finish()
+
+    @staticmethod
+    def _example_center(ex, center):
+        """Centre of the last coordinate set, unless every set is empty or one is given
+        (src/grid_maker.cpp:120-133)."""
+        if center is not None:
+            c = _to_float3(center)
+            if not math.isinf(c.x):
+                return c
+        c = float3()
+        for cs in reversed(ex.coord_sets):
+            c = float3()
+            if cs.size():
+                c = ex.coord_sets[-1].center()
+                break
+        return c
+
+    def _forward_example(self, ex, transform, grid):
+        # src/grid_maker.cpp:108-115: merge (a copy), transform the copy, grid about the centre
+        c = ex.merge_coordinates()
+        g = _unwrap(grid)
+        if c.max_type != tuple(g.shape)[0]:
+            raise IndexError("Incorrect number of channels in output grid: %d vs %d"
+                             % (c.max_type, tuple(g.shape)[0]))
+        if not _is_host(g):
+            c.togpu()
+        transform.forward(c, c)
+        self.forward(transform.get_rotation_center(), c, grid)
+
+    def _forward_examples(self, examples, grid, random_translation, random_rotation):
+        """include/libmolgrid/grid_maker.h:194-201.  The transforms are drawn example by example,
+        as the reference's loop does; index-typed examples are then packed and gridded with one
+        transform launch and one forward launch for the whole batch."""
+        g = _unwrap(grid)
+        if len(examples) != tuple(g.shape)[0]:
+            raise IndexError("output grid dimension does not match size of example vector")
+        transforms = [Transform(self._example_center(ex, None), random_translation,
+                                random_rotation) for ex in examples]
+        merged = [ex.merge_coordinates() for ex in examples]
+        packable = len(examples) > 1 and len(tuple(g.shape)) == 5 and all(
+            m.size() > 0 and m.type_index.size() > 0 and m.max_type == tuple(g.shape)[1]
+            for m in merged) and not self._p.radii_type_indexed
+        if not packable:
+            for i, (ex, t) in enumerate(zip(examples, transforms)):
+                self._forward_example(ex, t, g[i])
+            return
+        offsets = np.zeros(len(merged) + 1, np.int64)
+        offsets[1:] = np.cumsum([m.size() for m in merged])
+        coords = np.concatenate([m.coords.tonumpy() for m in merged])
+        types = np.concatenate([m.type_index.tonumpy() for m in merged])
+        radii = np.concatenate([m.radii.tonumpy() for m in merged])
+        quats = np.asarray([t.get_quaternion().as_tuple() for t in transforms], np.float32)
+        centers = np.asarray([tuple(t.get_rotation_center()) for t in transforms], np.float32)
+        shifts = np.asarray([tuple(t.get_translation()) for t in transforms], np.float32)
+        batch = AtomBatch(offsets)
+        dev_coords = torch.from_numpy(coords).to(_device())
+        transform_batch(batch, quats, centers, shifts, dev_coords, dev_coords)
+        self.forward_batch(batch, centers, dev_coords, torch.from_numpy(types).to(_device()),
+                           torch.from_numpy(radii).to(_device()), grid)
 
     def _forward_padded(self, centers, coords, types, radii, grid):
         # include/libmolgrid/grid_maker.h:265-301; one centre for all examples is accepted too

@@ -1,0 +1,132 @@
+"""Examples through the gridding calls (include/libmolgrid/grid_maker.h:153-201): an example is
+merged, transformed and gridded about the transform's centre; a batch of examples draws its
+transforms example by example and is gridded with one launch."""
+import numpy as np
+import pytest
+import torch
+from pytest import approx
+
+import oracle
+from util import assert_close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def molgrid():
+    import libmolgrid_amd
+    return libmolgrid_amd
+
+
+def make_example(molgrid, seed, nrec=60, nlig=9):
+    rng = np.random.default_rng(seed)
+    ex = molgrid.Example()
+    rec = molgrid.CoordinateSet(rng.uniform(-6, 6, (nrec, 3)).astype(np.float32),
+                                rng.integers(0, 5, nrec).astype(np.float32),
+                                rng.uniform(1.2, 2.0, nrec).astype(np.float32), 5)
+    lig = molgrid.CoordinateSet(rng.uniform(-2, 3, (nlig, 3)).astype(np.float32),
+                                rng.integers(0, 3, nlig).astype(np.float32),
+                                rng.uniform(1.2, 2.0, nlig).astype(np.float32), 3)
+    ex.coord_sets = [rec, lig]
+    ex.labels = [float(seed % 2), 0.25 * seed]
+    return ex
+
+
+def test_coordset_transform_on_device(molgrid):
+    """test/test_coordinateset.py:69-88"""
+    coords = np.array([[1, 0, -1], [1, 3, -1], [1, 0, -1]], np.float32)
+    c = molgrid.CoordinateSet(coords, np.array([3, 2, 1], np.float32),
+                              np.array([1.5, 1.5, 1.0], np.float32), 4)
+    t = molgrid.Transform(molgrid.Quaternion(), (0, 0, 0), (-1, 0, 1))
+    t.forward(c, c)
+    assert c.coords[1, 1] == 3.0
+    assert np.sum(c.coords.tonumpy()) == approx(3.0)
+    c.togpu()
+    assert c.coords.ongpu() and c.radii.ongpu()
+    t.backward(c, c)
+    assert np.array_equal(c.coords.tonumpy(), coords)
+    cd = molgrid.CoordinateSet(dev(coords), dev(np.array([3, 2, 1], np.float32)),
+                               dev(np.array([1.5, 1.5, 1.0], np.float32)), 4)
+    assert cd.coords.ongpu() and cd.size() == 3
+
+
+def test_forward_example_with_transform(molgrid):
+    ex = make_example(molgrid, 3)
+    gm = molgrid.GridMaker(0.5, 11.5)
+    q = np.random.default_rng(1).normal(size=4)
+    T = molgrid.Transform(molgrid.Quaternion(*(q / np.linalg.norm(q))), (0.5, -0.25, 1.0),
+                          (0.3, 0.2, -0.1))
+    out = torch.empty(gm.grid_dimensions(8), device="cuda")
+    gm.forward(ex, T, out)
+    m = ex.merge_coordinates()
+    moved = oracle.transform_forward(q / np.linalg.norm(q), (0.5, -0.25, 1.0), (0.3, 0.2, -0.1),
+                                     m.coords.tonumpy())
+    ref = oracle.GridMaker(0.5, 11.5).forward((0.5, -0.25, 1.0), moved, m.type_index.tonumpy(),
+                                              m.radii.tonumpy(), 8)
+    assert_close(out.cpu().numpy(), ref, what="forward(example, transform)")
+    assert np.array_equal(ex.coord_sets[0].coords.tonumpy(),
+                          make_example(molgrid, 3).coord_sets[0].coords.tonumpy())   # untouched
+    host = molgrid.MGrid4f(*gm.grid_dimensions(8))
+    gm.forward(ex, T, host.cpu())
+    assert np.array_equal(host.tonumpy(), out.cpu().numpy())
+    with pytest.raises(IndexError):
+        gm.forward(ex, T, torch.empty(gm.grid_dimensions(7), device="cuda"))
+
+
+def test_forward_example_default_center(molgrid):
+    """Without a centre the grid sits on the centre of the last coordinate set."""
+    ex = make_example(molgrid, 5)
+    gm = molgrid.GridMaker(0.5, 11.5)
+    out = torch.empty(gm.grid_dimensions(8), device="cuda")
+    gm.forward(ex, out)
+    m = ex.merge_coordinates()
+    center = tuple(ex.coord_sets[1].center())
+    ref = oracle.GridMaker(0.5, 11.5).forward(center, m.coords.tonumpy(), m.type_index.tonumpy(),
+                                              m.radii.tonumpy(), 8)
+    assert_close(out.cpu().numpy(), ref, what="forward(example)")
+    out2 = torch.empty_like(out)
+    gm.forward(ex, out2, center=(0, 0, 0))
+    ref2 = oracle.GridMaker(0.5, 11.5).forward((0, 0, 0), m.coords.tonumpy(),
+                                               m.type_index.tonumpy(), m.radii.tonumpy(), 8)
+    assert_close(out2.cpu().numpy(), ref2, what="forward(example, center)")
+
+
+def test_forward_batch_of_examples(molgrid):
+    """One launch for the batch gives what the reference's loop over the examples gives: the same
+    random transforms in the same order, the same grids bit for bit."""
+    batch = molgrid.ExampleVec([make_example(molgrid, s, nrec=40 + 7 * s) for s in range(6)])
+    gm = molgrid.GridMaker(0.5, 11.5)
+    out = torch.empty((6,) + gm.grid_dimensions(8), device="cuda")
+    molgrid.set_random_seed(17)
+    gm.forward(batch, out, random_translation=2.0, random_rotation=True)
+    one = torch.empty_like(out)
+    molgrid.set_random_seed(17)
+    for i, ex in enumerate(batch):
+        gm.forward(ex, one[i], random_translation=2.0, random_rotation=True)
+    assert torch.equal(out, one)
+    assert float(out.sum()) > 0
+    # no randomness: each grid is the example about its ligand's centre
+    gm.forward(batch, out)
+    m = batch[2].merge_coordinates()
+    ref = oracle.GridMaker(0.5, 11.5).forward(tuple(batch[2].coord_sets[1].center()),
+                                              m.coords.tonumpy(), m.type_index.tonumpy(),
+                                              m.radii.tonumpy(), 8)
+    assert_close(out[2].cpu().numpy(), ref, what="forward(batch)")
+    with pytest.raises(IndexError):
+        gm.forward(batch, torch.empty((5,) + gm.grid_dimensions(8), device="cuda"))
+    labels = torch.empty((6, 2), device="cuda")
+    batch.extract_labels(labels)
+    assert labels[3].tolist() == [1.0, 0.75]
+
+
+def test_backward_with_coordinate_set(molgrid):
+    ex = make_example(molgrid, 8)
+    m = ex.merge_coordinates()
+    gm = molgrid.GridMaker(0.5, 11.5)
+    diff = torch.randn(gm.grid_dimensions(8), device="cuda")
+    grads = molgrid.MGrid2f(m.size(), 3)
+    gm.backward((0, 0, 0), m, diff, grads.gpu())
+    direct = torch.empty((m.size(), 3), device="cuda")
+    gm.backward((0, 0, 0), dev(m.coords.tonumpy()), dev(m.type_index.tonumpy()),
+                dev(m.radii.tonumpy()), diff, direct)
+    assert np.array_equal(grads.tonumpy(), direct.cpu().numpy())
