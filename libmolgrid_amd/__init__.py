@@ -10,6 +10,9 @@ from .gridding import (AtomBatch, CoordinateSet, Example, ExampleVec, GridInterp
                        Quaternion, Transform, float3, set_random_seed, transform_batch)
 
 from .grids import *  # noqa: F401,F403,E402  (Grid1f .. Grid8dCUDA, MGrid1f .. MGrid8d, tonumpy)
+from .typers import *  # noqa: F401,F403,E402
+from .providers import *  # noqa: F401,F403,E402
+from .grid_io import *  # noqa: F401,F403,E402
 from .torch_bindings import (BatchedCoords2GridFunction, Coords2Grid, Coords2GridFunction,  # noqa: F401,E402
                              Grid2CoordsGradientFunction)
 

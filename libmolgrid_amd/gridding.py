@@ -770,7 +770,8 @@ class Example(object):
         coords, types, radii, offset = [], [], [], 0
         for cs in sets:
             n = cs.size()
-            tv = cs.type_vector.tonumpy().reshape(n, -1)
+            tv = cs.type_vector.tonumpy()
+            tv = tv.reshape(n, tv.shape[1] if tv.ndim == 2 else 0)
             if offset + tv.shape[1] > maxt and n > 0:
                 raise RuntimeError("Incompatible vector sizes in merge_coordinates")
             block = np.zeros((n, maxt), np.float32)
@@ -885,6 +886,15 @@ class ExampleVec(list):
             o.copy_(torch.from_numpy(vals))
         else:
             o[...] = vals
+
+    def sum_types(self, out, unique_types=True):
+        """out[i, :] = type sums of example i (python/bindings.in.cpp:384-393)."""
+        o = _unwrap(out)
+        if tuple(o.shape)[0] != len(self):
+            raise ValueError("Size of example vector does not match sum grid: %d vs %d"
+                             % (len(self), tuple(o.shape)[0]))
+        for i, ex in enumerate(self):
+            ex.sum_types(o[i], unique_types)
 
     def extract_label(self, labelpos, out):
         """out[i] = label `labelpos` of example i (src/example.cpp:278-299)."""

@@ -130,3 +130,62 @@ def test_backward_with_coordinate_set(molgrid):
     gm.backward((0, 0, 0), dev(m.coords.tonumpy()), dev(m.type_index.tonumpy()),
                 dev(m.radii.tonumpy()), diff, direct)
     assert np.array_equal(grads.tonumpy(), direct.cpu().numpy())
+
+
+def test_training_loop_from_example_provider(molgrid):
+    """The loop of the reference's README: a provider over an example list, a batch gridded into a
+    device tensor with random rotations and translations, labels extracted to the device
+    (test/test_example_provider.py:74-123, test/test_gridmaker.py:86-100)."""
+    import os
+    datadir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "molgrid_data")
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs", balanced=True, shuffle=True)
+    molgrid.set_random_seed(0)
+    e.populate(datadir + "/small.types")
+    for part in (e.provider.actives, e.provider.decoys):      # structure files among the fixtures
+        part.all = [r for r in part.all
+                    if all(os.path.exists(datadir + "/structs/" + f) for f in r.files)]
+        assert len(part.all) >= 12
+    gmaker = molgrid.GridMaker()
+    dims = gmaker.grid_dimensions(e.num_types())
+    assert dims == (28, 48, 48, 48)
+    batch_size = 8
+    tensor = torch.zeros((batch_size,) + dims, dtype=torch.float32, device="cuda")
+    labels = torch.zeros(batch_size, dtype=torch.float32, device="cuda")
+    for _ in range(3):
+        batch = e.next_batch(batch_size)
+        gmaker.forward(batch, tensor, random_translation=2.0, random_rotation=True)
+        batch.extract_label(0, labels)
+        assert labels.tolist() == [1.0, 0.0] * 4
+        per_example = tensor.reshape(batch_size, -1).sum(1)
+        assert bool((per_example > 100).all())
+    # without randomness the grid is the oracle's grid about the ligand's centre
+    ex = batch[0]
+    out = torch.empty(dims, device="cuda")
+    gmaker.forward(ex, out)
+    m = ex.merge_coordinates()
+    ref = oracle.GridMaker(0.5, 23.5).forward(tuple(ex.coord_sets[1].center()), m.coords.tonumpy(),
+                                              m.type_index.tonumpy(), m.radii.tonumpy(), 28)
+    assert_close(out.cpu().numpy(), ref, what="example from the provider")
+
+
+def test_vector_typed_examples_with_type_radii(molgrid):
+    """test/test_example_provider.py:236-265: one-hot type vectors with radii per type."""
+    import os
+    datadir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "molgrid_data")
+    e = molgrid.ExampleProvider(molgrid.NullIndexTyper(), molgrid.defaultGninaLigandTyper,
+                                data_root=datadir + "/structs", make_vector_types=True)
+    e.populate(datadir + "/ligonly.types")
+    b = e.next_batch(10)
+    gmaker = molgrid.GridMaker(dimension=23.5, radius_type_indexed=True)
+    shape = gmaker.grid_dimensions(molgrid.defaultGninaLigandTyper.num_types())
+    mgrid = molgrid.MGrid5f(10, *shape)
+    gmaker.forward(b, mgrid.gpu())
+    # the same atoms through index types and per-atom radii
+    e2 = molgrid.ExampleProvider(molgrid.NullIndexTyper(), molgrid.defaultGninaLigandTyper,
+                                 data_root=datadir + "/structs")
+    e2.populate(datadir + "/ligonly.types")
+    b2 = e2.next_batch(10)
+    plain = torch.empty((10,) + shape, device="cuda")
+    molgrid.GridMaker(dimension=23.5).forward(b2, plain)
+    assert_close(mgrid.tonumpy(), plain.cpu().numpy(), what="type-indexed radii vs per-atom radii")
+    assert float(plain.sum()) > 0
