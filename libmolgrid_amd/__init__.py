@@ -14,7 +14,11 @@ from .typers import *  # noqa: F401,F403,E402
 from .providers import *  # noqa: F401,F403,E402
 from .grid_io import *  # noqa: F401,F403,E402
 from .torch_bindings import (BatchedCoords2GridFunction, Coords2Grid, Coords2GridFunction,  # noqa: F401,E402
-                             Grid2CoordsGradientFunction)
+                             Grid2CoordsGradientFunction, MolIterDataset, MolMapDataset,
+                             make_grid_ndarray, make_grid_tensor, tensor_as_grid)
+
+GridMaker.make_tensor = make_grid_tensor
+GridMaker.make_ndarray = make_grid_ndarray
 
 __version__ = "0.1.0"
 

@@ -738,7 +738,59 @@ class ExampleProvider(object):
             c._restore(s)
 
 
-__all__ = ["IterationScheme", "ExampleProviderSettings", "ExampleRef", "ExampleProvider",
+class ExampleDataset(object):
+    """The examples of a list by position, in file order (include/libmolgrid/example_dataset.h)."""
+
+    def __init__(self, *args, **kw):
+        args = list(args)
+        settings = ExampleProviderSettings()
+        if args and isinstance(args[0], ExampleProviderSettings):
+            settings = args.pop(0).copy()
+        settings.update(kw)
+        self.init_settings = settings
+        self.provider = UniformExampleRefProvider(ExampleProviderSettings())
+        typers = args or [defaultGninaReceptorTyper, defaultGninaLigandTyper]
+        molcaches = [settings.recmolcache, settings.ligmolcache] if not args else []
+        self.extractor = ExampleExtractor(settings, typers, molcaches)
+
+    def populate(self, file_name, num_labels=-1):
+        names = [file_name] if isinstance(file_name, str) else list(file_name)
+        for name in names:
+            try:
+                f = open(name)
+            except OSError:
+                raise ValueError("Could not open file " + name)
+            with f:
+                self.provider.populate(f, num_labels)
+
+    def __len__(self):
+        return self.provider.size()
+
+    def size(self):
+        return self.provider.size()
+
+    def __getitem__(self, idx):
+        n = self.provider.size()
+        if idx < 0:
+            idx += n
+        if not 0 <= idx < n:
+            raise IndexError("Invalid index: %d" % idx)
+        return self.extractor.extract(self.provider[idx])
+
+    def num_labels(self):
+        return self.provider.num_labels()
+
+    def settings(self):
+        return self.init_settings
+
+    def num_types(self):
+        return self.extractor.num_types()
+
+    def get_type_names(self):
+        return self.extractor.get_type_names()
+
+
+__all__ = ["IterationScheme", "ExampleProviderSettings", "ExampleRef", "ExampleProvider", "ExampleDataset",
            "ExampleExtractor", "CoordCache", "UniformExampleRefProvider",
            "BalancedExampleRefProvider", "ReceptorStratifiedExampleRefProvider",
            "ValueStratifiedExampleRefProvider", "GroupedExampleRefProvider"]

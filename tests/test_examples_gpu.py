@@ -189,3 +189,56 @@ def test_vector_typed_examples_with_type_radii(molgrid):
     molgrid.GridMaker(dimension=23.5).forward(b2, plain)
     assert_close(mgrid.tonumpy(), plain.cpu().numpy(), what="type-indexed radii vs per-atom radii")
     assert float(plain.sum()) > 0
+
+
+def test_datasets_grid_like_the_provider(molgrid):
+    """test/test_example_provider.py:357-492: padded batches from the two datasets gridded with the
+    tensor overload equal the provider's examples gridded directly; random transforms in a dataset
+    are rigid motions about the last coordinate set's centre."""
+    import os
+    datadir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "molgrid_data")
+    fname = datadir + "/small.types"
+    bsize = 8
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs", default_batch_size=bsize)
+    e.populate(fname)
+    m = molgrid.MolIterDataset(fname, data_root=datadir + "/structs", default_batch_size=bsize)
+    it = iter(m)
+    next(it)
+    lengths, center, coords, types, radii, labels = next(it)
+    e.next_batch()
+    ex = e.next_batch()
+    gmaker = molgrid.GridMaker()
+    shape = gmaker.grid_dimensions(e.num_types())
+    mgridg = molgrid.MGrid5f(bsize, *shape)
+    gmaker.forward(center.cuda(), coords.cuda(), types.cuda(), radii.cuda(), mgridg.gpu())
+    egrid = molgrid.MGrid5f(bsize, *shape)
+    gmaker.forward(ex, egrid.gpu())
+    np.testing.assert_allclose(mgridg.tonumpy(), egrid.tonumpy(), atol=1e-5)
+    assert float(egrid.tonumpy().sum()) > 1000
+
+    mm = molgrid.MolMapDataset(fname, data_root=datadir + "/structs")
+    loader = torch.utils.data.DataLoader(mm, batch_size=bsize,
+                                         collate_fn=molgrid.MolMapDataset.collateMolDataset)
+    it = iter(loader)
+    next(it)
+    lengths, center, coords, types, radii, labels = next(it)
+    mgrid = molgrid.MGrid5f(bsize, *shape)
+    gmaker.forward(center.cuda(), coords.cuda(), types.cuda(), radii.cuda(), mgrid.gpu())
+    np.testing.assert_allclose(mgrid.tonumpy(), egrid.tonumpy(), atol=1e-5)
+    one = gmaker.make_tensor(tuple(ex[2].coord_sets[-1].center()), ex[2].merge_coordinates())
+    assert tuple(one.shape) == shape and one.is_cuda
+    np.testing.assert_allclose(one.cpu().numpy(), egrid.tonumpy()[2], atol=1e-5)
+    arr = gmaker.make_ndarray(tuple(ex[2].coord_sets[-1].center()), ex[2].merge_coordinates())
+    np.testing.assert_allclose(arr, egrid.tonumpy()[2], atol=1e-5)
+
+    mlength, mcenter, mcoords, mtypes, mradii, mlabels = mm[10]
+    molgrid.set_random_seed(3)
+    r = molgrid.MolMapDataset(fname, data_root=datadir + "/structs", random_translation=2.0,
+                              random_rotation=True)
+    rl, rc, rcoords, rtypes, rradii, rlabels = r[10]
+    np.testing.assert_allclose(rc, mcenter)
+    assert rtypes.tolist() == mtypes.tolist() and rlabels.tolist() == mlabels.tolist()
+    d0 = torch.cdist(mcoords[:20], mcoords[:20])
+    d1 = torch.cdist(rcoords[:20], rcoords[:20])
+    np.testing.assert_allclose(d0, d1, atol=2e-3)
+    assert float((rcoords - mcoords).abs().max()) > 0.5

@@ -437,3 +437,120 @@ def test_write_map(molgrid, tmp_path):
     assert lines[3] == "SPACING 0.375" and lines[4] == "NELEMENTS 2 2 2" and lines[5] == "CENTER 0 1 2"
     assert lines[6] == "0" and lines[7] == "%.5g" % g[1, 0, 0] and lines[9] == "%.5g" % g[0, 1, 0]
     assert len(lines) == 6 + 27 + 1
+
+
+# ---- datasets over example lists (test/test_example_provider.py:357-492) --------------------
+def test_example_dataset_and_map_dataset(molgrid):
+    """test/test_example_provider.py:357-406 on the examples whose structure files are among the
+    fixtures (the first 120 lines of the list)."""
+    fname = datadir + "/small.types"
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs")
+    e.populate(fname)
+    m = molgrid.MolMapDataset(fname, data_root=datadir + "/structs")
+    assert len(m) == 1000
+    assert m.examples.num_labels() == 3 and m.examples.num_types() == 28
+    ex = e.next()
+    coordinates = ex.merge_coordinates()
+    length, center, coords, types, radii, labels = m[0]
+    assert length == 1791 and list(center.shape) == [3]
+    np.testing.assert_allclose(center, list(ex.coord_sets[-1].center()))
+    np.testing.assert_allclose(coords, coordinates.coords.tonumpy())
+    np.testing.assert_allclose(types, coordinates.type_index.tonumpy())
+    np.testing.assert_allclose(radii, coordinates.radii.tonumpy())
+    assert len(labels) == 3 and labels[0] == 1
+    np.testing.assert_allclose(labels[1], 6.05)
+    np.testing.assert_allclose(labels[-1], 0.162643)
+    ref = m.examples.provider[len(m) - 1]                         # the last line of the list
+    assert ref.labels[0] == 0 and ref.labels[1] == approx(-10.3)
+    with pytest.raises(IndexError):
+        m.examples[1000]
+
+    loader = torch.utils.data.DataLoader(m, batch_size=8,
+                                         collate_fn=molgrid.MolMapDataset.collateMolDataset)
+    it = iter(loader)
+    next(it)
+    lengths, center, coords, types, radii, labels = next(it)
+    for t in (lengths, center, coords, types, radii, labels):
+        assert t.shape[0] == 8
+    mlength, mcenter, mcoords, mtypes, mradii, mlabels = m[10]
+    n = int(lengths[2])
+    assert n == mlength
+    np.testing.assert_allclose(center[2], mcenter)
+    np.testing.assert_allclose(coords[2][:n], mcoords)
+    np.testing.assert_allclose(types[2][:n], mtypes)
+    np.testing.assert_allclose(radii[2][:n], mradii)
+    assert float(radii[2][n:].abs().sum()) == 0                    # padded with zeros
+    assert labels[2].tolist() == mlabels.tolist()
+
+
+def test_iterable_dataset_and_pickling(molgrid):
+    """test/test_example_provider.py:408-470 (single process) and the datasets' pickling."""
+    import pickle
+    fname = datadir + "/small.types"
+    bsize = 25
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs", default_batch_size=bsize)
+    e.populate(fname)
+    m = molgrid.MolIterDataset(fname, data_root=datadir + "/structs", default_batch_size=bsize)
+    it = iter(m)
+    coordinates = e.next().merge_coordinates()
+    lengths, centers, coords, types, radii, labels = next(it)
+    assert list(centers.shape) == [bsize, 3]
+    n = int(lengths[0])
+    np.testing.assert_allclose(coords[0, :n, :], coordinates.coords.tonumpy())
+    np.testing.assert_allclose(types[0, :n], coordinates.type_index.tonumpy())
+    np.testing.assert_allclose(radii[0, :n], coordinates.radii.tonumpy())
+    assert len(labels) == bsize and len(labels[0]) == 3 and labels[0, 0] == 1
+    np.testing.assert_allclose(labels[0, 1], 6.05)
+    np.testing.assert_allclose(labels[0, -1], 0.162643)
+
+    m.examples.reset()
+    loader = torch.utils.data.DataLoader(m, batch_size=None)
+    it = iter(loader)
+    next(it)
+    lengths, center, coords, types, radii, labels = next(it)
+    for t in (lengths, center, coords, types, radii, labels):
+        assert t.shape[0] == bsize
+    e.reset()
+    e.next_batch()
+    ex = e.next_batch()
+    coordinates = ex[2].merge_coordinates()
+    n = int(lengths[2])
+    np.testing.assert_allclose(center[2], np.array(list(ex[2].coord_sets[-1].center())))
+    np.testing.assert_allclose(coords[2, :n], coordinates.coords.tonumpy())
+    np.testing.assert_allclose(types[2, :n], coordinates.type_index.tonumpy())
+    np.testing.assert_allclose(radii[2, :n], coordinates.radii.tonumpy())
+    assert labels[2].tolist() == [approx(v) for v in ex[2].labels]
+
+    with pytest.raises(NotImplementedError):
+        len(m)                                                     # continuous: no length
+    small = molgrid.MolIterDataset(fname, data_root=datadir + "/structs", default_batch_size=bsize,
+                                   iteration_scheme=molgrid.IterationScheme.SmallEpoch)
+    assert len(small) == 1000 // bsize
+    large = molgrid.MolIterDataset(fname, data_root=datadir + "/structs", default_batch_size=30,
+                                   iteration_scheme=molgrid.IterationScheme.LargeEpoch)
+    assert len(large) == 34
+
+    again = pickle.loads(pickle.dumps(small))
+    assert len(again) == len(small) and again.examples.settings().default_batch_size == bsize
+    a, b = next(iter(again)), next(iter(small))
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    mm = pickle.loads(pickle.dumps(molgrid.MolMapDataset(fname, data_root=datadir + "/structs")))
+    assert len(mm) == 1000 and mm[3][0] == mm[3][2].shape[0]
+    typed = molgrid.MolMapDataset(fname, data_root=datadir + "/structs",
+                                  typers=(molgrid.defaultGninaReceptorTyper,
+                                          molgrid.defaultGninaLigandTyper))
+    with pytest.raises(NotImplementedError):
+        pickle.dumps(typed)
+
+
+def test_tensor_as_grid_and_make_ndarray(molgrid):
+    """python/torch_bindings.py:9-43"""
+    t = torch.zeros(3, 4, 5)
+    g = molgrid.tensor_as_grid(t)
+    assert type(g).__name__ == "Grid3f" and g.shape == (3, 4, 5)
+    assert type(molgrid.tensor_as_grid(t.double()[0])).__name__ == "Grid2d"
+    with pytest.raises(ValueError):
+        molgrid.tensor_as_grid(torch.zeros(3, dtype=torch.int32))
+    assert molgrid.GridMaker.make_ndarray is molgrid.make_grid_ndarray
+    assert molgrid.GridMaker.make_tensor is molgrid.make_grid_tensor
