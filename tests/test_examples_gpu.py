@@ -242,3 +242,44 @@ def test_datasets_grid_like_the_provider(molgrid):
     d1 = torch.cdist(rcoords[:20], rcoords[:20])
     np.testing.assert_allclose(d0, d1, atol=2e-3)
     assert float((rcoords - mcoords).abs().max()) > 0.5
+
+
+def test_training_a_small_network_on_gridded_batches(molgrid):
+    """The reference's end-to-end training test (test/test_torch_cnn.py) on the examples whose
+    structure files are among the fixtures: balanced, shuffled batches gridded straight into a
+    device tensor, labels extracted, a small network trained until it separates the classes.
+    (Pooling and linear layers instead of the reference's 3-D convolutions keep the test short.)"""
+    import os
+    import torch.nn as nn
+    import torch.nn.functional as F
+    datadir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "molgrid_data")
+    molgrid.set_random_seed(0)
+    torch.manual_seed(0)
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs", balanced=True, shuffle=True)
+    e.populate(datadir + "/small.types")
+    for part in (e.provider.actives, e.provider.decoys):
+        part.all = [r for r in part.all
+                    if all(os.path.exists(datadir + "/structs/" + f) for f in r.files)][:12]
+        assert len(part.all) == 12
+    gmaker = molgrid.GridMaker()
+    dims = gmaker.grid_dimensions(e.num_types())
+    batch_size = 24
+    model = nn.Sequential(nn.MaxPool3d(4), nn.Flatten(),
+                          nn.Linear(dims[0] * (dims[1] // 4) ** 3, 64), nn.ReLU(),
+                          nn.Linear(64, 2)).to("cuda")
+    optimizer = torch.optim.SGD(model.parameters(), lr=0.01, momentum=0.9)
+    input_tensor = torch.zeros((batch_size,) + dims, dtype=torch.float32, device="cuda")
+    float_labels = torch.zeros(batch_size, dtype=torch.float32)
+    losses = []
+    for _ in range(60):
+        batch = e.next_batch(batch_size)
+        gmaker.forward(batch, input_tensor, 0, random_rotation=False)
+        batch.extract_label(0, float_labels)
+        labels = float_labels.long().to("cuda")
+        assert int(labels.sum()) == batch_size // 2                # balanced
+        optimizer.zero_grad()
+        loss = F.cross_entropy(model(input_tensor), labels)
+        loss.backward()
+        optimizer.step()
+        losses.append(loss.item())
+    assert np.mean(losses[-5:]) < 0.4 < losses[0]

@@ -122,3 +122,36 @@ def test_conversion_rules(molgrid):
     sub[3, 4] = 9.0
     assert m[1, 2, 3, 4] == 9.0 and sub.shape == (4, 5)
     assert np.asarray(m).shape == (2, 3, 4, 5)
+
+
+def _filled_mgrids(molgrid):
+    mg2 = molgrid.MGrid2f(3, 4)
+    mg3 = molgrid.MGrid3d(3, 4, 2)
+    for i in range(3):
+        for j in range(4):
+            mg2[i, j] = i * j + 1
+            for k in range(2):
+                mg3[i, j, k] = i * j + 1 + k
+    return mg2, mg3
+
+
+def test_mgrid_copyto_and_copyfrom_tensor(molgrid):
+    """test/test_torch.py:9-37, 55-76"""
+    import torch
+    mg2, mg3 = _filled_mgrids(molgrid)
+    t2 = torch.zeros(3, 4)
+    t3 = torch.zeros(3, 4, 2, dtype=torch.float64)
+    assert mg2.copyTo(t2) == 12 and mg3.copyTo(t3) == 24
+    for i in range(3):
+        for j in range(4):
+            assert t2[i, j] == i * j + 1
+            for k in range(2):
+                assert t3[i, j, k] == i * j + 1 + k
+    b2, b3 = molgrid.MGrid2f(3, 4), molgrid.MGrid3d(3, 4, 2)
+    b2.copyFrom(t2)
+    b3.copyFrom(t3)
+    for i in range(3):
+        for j in range(4):
+            assert b2[i, j] == i * j + 1
+            for k in range(2):
+                assert b3[i, j, k] == i * j + 1 + k

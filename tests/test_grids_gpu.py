@@ -132,3 +132,26 @@ def test_interpolater_takes_grids(molgrid):
     gi.forward(src.gpu(), molgrid.Transform(), dst.gpu())
     assert dst.ongpu()
     assert_close(dst.tonumpy(), src.tonumpy(), rtol=RTOL, atol=ATOL, what="identity resampling")
+
+
+def test_mgrid_copy_to_and_from_device_tensors(molgrid):
+    """test/test_torch.py:39-53, 78-99"""
+    mg2 = molgrid.MGrid2f(3, 4)
+    mg3 = molgrid.MGrid3d(3, 4, 2)
+    for i in range(3):
+        for j in range(4):
+            mg2[i, j] = i * j + 1
+            for k in range(2):
+                mg3[i, j, k] = i * j + 1 + k
+    t2 = torch.zeros(3, 4, device="cuda")
+    t3 = torch.zeros(3, 4, 2, dtype=torch.float64, device="cuda")
+    mg2.copyTo(t2)
+    mg3.copyTo(t3)
+    b2, b3 = molgrid.MGrid2f(3, 4), molgrid.MGrid3d(3, 4, 2)
+    b2.copyFrom(t2)
+    b3.copyFrom(t3)
+    for i in range(3):
+        for j in range(4):
+            assert t2[i, j] == i * j + 1 and b2[i, j] == i * j + 1
+            for k in range(2):
+                assert t3[i, j, k] == i * j + 1 + k and b3[i, j, k] == i * j + 1 + k

@@ -554,3 +554,20 @@ def test_tensor_as_grid_and_make_ndarray(molgrid):
         molgrid.tensor_as_grid(torch.zeros(3, dtype=torch.int32))
     assert molgrid.GridMaker.make_ndarray is molgrid.make_grid_ndarray
     assert molgrid.GridMaker.make_tensor is molgrid.make_grid_tensor
+
+
+def test_labels_into_tensors(molgrid):
+    """test/test_torch.py:102-126"""
+    e = molgrid.ExampleProvider(data_root=datadir + "/structs")
+    e.populate(datadir + "/small.types")
+    batch = e.next_batch(100)
+    assert e.num_labels() == 3
+    labels = torch.zeros((100, 3), dtype=torch.float32)
+    batch.extract_labels(labels)
+    label0 = torch.zeros(100, dtype=torch.float32)
+    batch.extract_label(0, label0)
+    assert label0[0] == 1 and labels[0, 0] == 1
+    assert float(labels[0][1]) == approx(6.05)
+    assert float(labels[0][2]) == approx(0.162643)
+    for i in range(100):
+        assert label0[i] == labels[i][0]
