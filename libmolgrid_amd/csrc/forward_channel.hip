@@ -1,0 +1,439 @@
+// Forward splat for index types, one channel at a time (GridMaker::forward,
+// src/grid_maker.cpp:160-211, src/grid_maker.cu:95-211).
+//
+// A workgroup owns three columns of 4 x 4 voxels in (x, y), consecutive in y, over a slab of up to
+// 48 voxels in z, like the column kernel of forward_index.hip, but walks the channels one after
+// the other: the atoms that can reach the columns are sorted by channel (stably, so each channel
+// keeps ascending atom order), the densities of one channel are summed in nine registers per lane
+// (one voxel in each of the wave's nine 4x4x4 blocks, in atom order), put into an LDS stage that
+// holds the three columns of that channel, and written out as whole z rows.  Only the sums of the
+// current channel live in registers, so the kernel needs few of them and many waves fit a CU.
+//
+// Every global access goes through buffer instructions with the extent of the array they address,
+// so an index outside it reads zero or is dropped.
+#include "kernels.h"
+#include "splat_common.h"
+
+namespace mg {
+namespace {
+
+constexpr int kColXY = 4;                        // column footprint in x and y
+constexpr int kCols = 3;                         // columns per workgroup
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kBlkPerWave = 3;                   // 4x4x4 blocks per wave and column
+constexpr int kSlabZ = kWaves * kBlkPerWave * 4; // 48
+constexpr int kBlocks = kCols * kBlkPerWave;     // blocks a wave owns
+constexpr int kPerRound = 7;                     // records per cull round: 7 x 9 blocks = 63 lanes
+constexpr int kRowPad = 52;                      // staged z row, padded against bank conflicts
+constexpr int kPlane = 16 * kRowPad;             // one staged column
+constexpr int kStage = kCols * kPlane;
+constexpr int kSuper = 2048;                     // atoms scanned per pass
+constexpr int kSeg = kSuper / kWaves;            // survivors kept per wave
+constexpr int kRecMax = 512;                     // records resident at a time
+constexpr int kSegs = kRecMax / kWave;           // 64-record pieces of the record array
+constexpr int kSortChannels = 64;                // channels the one-pass sort handles
+constexpr int kBufferFlags = 0x00020000;         // untyped 32-bit elements, no swizzle
+
+static_assert(kBlocks * kPerRound <= kWave, "one lane per (record, block) pair of a cull round");
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float uniform(float v) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void* p, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           (int)(bytes < 0xffffffffull ? bytes : 0xffffffffull),
+                                           kBufferFlags);
+}
+__device__ __forceinline__ float buffer_float(__amdgpu_buffer_rsrc_t r, int index) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, index * 4, 0, 0));
+}
+
+// LDS-only barrier: outstanding global stores are not waited for.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <bool BINARY>
+__global__ __launch_bounds__(kThreads) void splat_channel_kernel(
+    GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
+    const float* __restrict__ types, const float* __restrict__ radii, float* __restrict__ out,
+    int cols_per_side, int aligned_rows) {
+  __shared__ __align__(16) float s_stage[kStage];
+  __shared__ unsigned short s_idx[kWaves][kSeg];
+  __shared__ float4 s_rec[kRecMax];                // x, y, z, (ar^2 | 1/ar^2), sorted by channel
+  __shared__ int s_wcount[kWaves];
+  __shared__ int s_start[kSortChannels + 1];       // first record of each channel
+
+  // records per (64-record piece, channel) while the records are sorted: the stage is not in use then
+  int (*s_cnt)[kSortChannels] = reinterpret_cast<int (*)[kSortChannels]>(s_stage);
+  static_assert(kSegs * kSortChannels <= kStage, "the counts fit the stage");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int b = example_for_slot(batch, blockIdx.y, gridDim.y, lane);
+  int begin, end;
+  example_range(batch, b, begin, end);
+  const int natoms = max(end - begin, 0);          // atoms are numbered from the example's first
+  const float3 center = load3(centers, b);
+  const float ox = uniform(center.x - g.half_dimension);
+  const float oy = uniform(center.y - g.half_dimension);
+  const float oz = uniform(center.z - g.half_dimension);
+  const int dim = g.dim;
+  const int ntypes = g.ntypes;
+
+  const __amdgpu_buffer_rsrc_t coords_buf = buffer_of(coords + (size_t)begin * 3, (size_t)natoms * 12);
+  const __amdgpu_buffer_rsrc_t radii_buf = buffer_of(radii + begin, (size_t)natoms * 4);
+  const __amdgpu_buffer_rsrc_t types_buf = buffer_of(types + begin, (size_t)natoms * 4);
+  const size_t chan_stride = (size_t)dim * dim * dim;
+  // the grids of this example; the host has checked that they fit a buffer's 32-bit extent
+  const __amdgpu_buffer_rsrc_t out_buf =
+      buffer_of(out + (size_t)b * ntypes * chan_stride, (size_t)ntypes * chan_stride * 4);
+
+  // which three columns and which z slab
+  const int groups_per_row = (cols_per_side + kCols - 1) / kCols;
+  const int ngroups = cols_per_side * groups_per_row;
+  const int slab = blockIdx.x / ngroups;
+  const int grp = blockIdx.x - slab * ngroups;
+  const int x0 = (grp / groups_per_row) * kColXY;
+  const int gy0 = (grp % groups_per_row) * (kColXY * kCols);
+  const int z0 = slab * kSlabZ;
+  const int zend = min(z0 + kSlabZ, dim);          // exclusive
+
+  // box of the whole group (first/last voxel centre inside the grid)
+  const float clx = uniform(grid_coord(ox, x0, g.resolution));
+  const float chx = uniform(grid_coord(ox, min(x0 + kColXY, dim) - 1, g.resolution));
+  const float gly = uniform(grid_coord(oy, gy0, g.resolution));
+  const float ghy = uniform(grid_coord(oy, min(gy0 + kColXY * kCols, dim) - 1, g.resolution));
+  const float clz = uniform(grid_coord(oz, z0, g.resolution));
+  const float chz = uniform(grid_coord(oz, zend - 1, g.resolution));
+
+  // the voxels this lane owns: one in each of the wave's nine blocks; a voxel outside the grid
+  // sits at infinity, where no atom reaches it
+  const int lx = lane >> 4, ly = (lane >> 2) & 3, lz = lane & 3;
+  const int vxi = x0 + lx;
+  const float vx = grid_coord(ox, vxi, g.resolution);
+  float vy[kCols], vz[kBlkPerWave];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    const int vyi = gy0 + c * kColXY + ly;
+    vy[c] = (vxi < dim && vyi < dim) ? grid_coord(oy, vyi, g.resolution) : INFINITY;
+  }
+#pragma unroll
+  for (int k = 0; k < kBlkPerWave; ++k) {
+    const int vzi = z0 + (wave * kBlkPerWave + k) * 4 + lz;
+    vz[k] = vzi < zend ? grid_coord(oz, vzi, g.resolution) : INFINITY;
+  }
+  const int stage_lane = (lx * 4 + ly) * kRowPad + wave * (kBlkPerWave * 4) + lz;
+
+  // the (record, block) pair this lane tests in a cull round, and that block's box
+  const int pair_block = lane / kPerRound;         // 0..8; lane 63 tests nothing
+  const int pair_rec = lane - pair_block * kPerRound;
+  float bly = INFINITY, bhy = INFINITY, blz = INFINITY, bhz = INFINITY;
+  if (pair_block < kBlocks) {
+    const int y0 = gy0 + (pair_block / kBlkPerWave) * kColXY;
+    const int zb = z0 + (wave * kBlkPerWave + pair_block % kBlkPerWave) * 4;
+    if (y0 < dim && zb < zend && x0 < dim) {
+      bly = grid_coord(oy, y0, g.resolution);
+      bhy = grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution);
+      blz = grid_coord(oz, zb, g.resolution);
+      bhz = grid_coord(oz, min(zb + 4, zend) - 1, g.resolution);
+    }
+  }
+
+  float quad_c = g.C;
+  asm volatile("" : "+v"(quad_c));          // vector register (an fma takes one scalar operand)
+  const float frm2 = uniform(g.frm * g.frm);
+  const float grm2 = uniform(g.grm * g.grm);
+  const float cull_mult = BINARY ? 1.0f : g.frm;   // support radius / ar
+
+  // fixed positions of this thread in the write-out of a channel (float4 granules of z rows)
+  constexpr int kItems = kCols * 16 * (kSlabZ / 4);                 // 576
+  constexpr int kPer = (kItems + kThreads - 1) / kThreads;          // 3
+  int st_lds[kPer], st_off[kPer], st_z[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    const int item = tid + k * kThreads;
+    const int col = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
+    const int gx = x0 + (row >> 2), gy = gy0 + col * kColXY + (row & 3), gz = z0 + f4 * 4;
+    st_lds[k] = min(col, kCols - 1) * kPlane + row * kRowPad + f4 * 4;
+    const bool ok = item < kItems && gx < dim && gy < dim && gz < zend;
+    st_z[k] = ok ? gz : dim;                                        // dim: nothing to write
+    st_off[k] = ok ? (int)((unsigned)((gx * dim + gy) * dim + gz) * 4u) : 0;
+  }
+
+  // One channel of the stage (or zeros) -> global memory as z rows.
+  auto store_channel = [&](int c, bool from_stage) {
+    const unsigned chan_off = (unsigned)c * (unsigned)(chan_stride * 4);   // < 4 GB in total
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      if (st_z[k] < dim) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (from_stage) {
+          v = *reinterpret_cast<const v4f*>(s_stage + st_lds[k]);
+        }
+        if (aligned_rows && st_z[k] + 3 < dim) {
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf,
+                                                 (int)(chan_off + (unsigned)st_off[k]), 0, 0);
+        } else {
+          const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (st_z[k] + t < dim)
+              __builtin_amdgcn_raw_buffer_store_b32(
+                  __builtin_bit_cast(unsigned, e[t]), out_buf,
+                  (int)(chan_off + (unsigned)st_off[k] + 4u * t), 0, 0);
+        }
+      }
+    }
+  };
+
+  int segstart[kWaves + 1];
+  int ncand = 0;
+
+  // ---- scan: atoms [s0, s1) against the group's box -> per-wave index segments --------------
+  // Each wave takes a contiguous quarter of the range and keeps up to kSeg survivors (offsets
+  // from s0 as 16-bit values, so s1 - s0 <= 65536).  `only` >= 0 keeps atoms of that channel
+  // only.  Returns false if a segment overflowed.
+  auto scan = [&](int s0, int s1, int only) -> bool {
+    const int quarter = (s1 - s0 + kWaves - 1) / kWaves;
+    int wcnt = 0;
+    const int wb = s0 + wave * quarter, we = min(s1, wb + quarter);
+    constexpr int U = 2;
+    for (int a0 = wb; a0 < we; a0 += kWave * U) {
+      float rr[U], cx[U], cy[U], cz[U], ty[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int a = min(a0 + u * kWave + lane, we - 1);
+        rr[u] = buffer_float(radii_buf, a);
+        cx[u] = buffer_float(coords_buf, 3 * a);
+        cy[u] = buffer_float(coords_buf, 3 * a + 1);
+        cz[u] = buffer_float(coords_buf, 3 * a + 2);
+        ty[u] = only >= 0 ? buffer_float(types_buf, a) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int a = a0 + u * kWave + lane;
+        const float reach = rr[u] * g.radius_scale * cull_mult;
+        bool p = (a < we) && box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy, chz) <=
+                                 reach * reach * kCullSlack;
+        if (only >= 0) p = p && floorf(ty[u]) == (float)only;
+        const unsigned long long m = __ballot(p);
+        const int pos = wcnt + __popcll(m & ((1ull << lane) - 1ull));
+        if (p && pos < kSeg) s_idx[wave][pos] = (unsigned short)(a - s0);
+        wcnt += __popcll(m);
+      }
+    }
+    if (lane == 0) s_wcount[wave] = wcnt;
+    __syncthreads();
+    segstart[0] = 0;
+    bool fits = true;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int c = __builtin_amdgcn_readfirstlane(s_wcount[w]);
+      fits = fits && c <= kSeg;
+      segstart[w + 1] = segstart[w] + min(c, kSeg);
+    }
+    ncand = segstart[kWaves];
+    lds_barrier();   // every wave has read the counts before any of them scans again
+    return fits;
+  };
+
+  // candidate gi of the current scan -> its atom; the record of that atom
+  auto atom_of = [&](int s0, int gi) -> int {
+    int w = 0;
+#pragma unroll
+    for (int k = 1; k < kWaves; ++k) w += (gi >= segstart[k]) ? 1 : 0;
+    return s0 + s_idx[w][min(gi - segstart[w], kSeg - 1)];
+  };
+  auto record_of = [&](int a) -> float4 {
+    const float ax = buffer_float(coords_buf, 3 * a), ay = buffer_float(coords_buf, 3 * a + 1),
+                az = buffer_float(coords_buf, 3 * a + 2);
+    float ar, ar2;
+    {
+#pragma clang fp contract(off)
+      ar = buffer_float(radii_buf, a) * g.radius_scale;
+      ar2 = ar * ar;
+    }
+    return make_float4(ax, ay, az, BINARY ? ar2 : 1.0f / ar2);
+  };
+
+  // the sums of the current channel at this lane's nine voxels
+  float acc[kBlocks];
+#pragma unroll
+  for (int q = 0; q < kBlocks; ++q) acc[q] = 0.f;
+  // sums -> stage (cleared for the next channel); the caller synchronises
+  auto stage_sums = [&]() {
+#pragma unroll
+    for (int q = 0; q < kBlocks; ++q) {
+      s_stage[stage_lane + (q / kBlkPerWave) * kPlane + (q % kBlkPerWave) * 4] = acc[q];
+      acc[q] = 0.f;
+    }
+  };
+
+  // ---- records [lo, hi) of s_rec, all of one channel, added to the sums -----------------------
+  // A cull round tests seven records against the wave's nine blocks, one pair per lane; the pairs
+  // that pass are taken block by block and, within a block, in record order.
+  auto splat_records = [&](int lo, int hi) {
+    for (int r0 = lo; r0 < hi; r0 += kPerRound) {
+      const int j = r0 + pair_rec;
+      const bool valid = pair_block < kBlocks && j < hi;
+      const float4 rec = s_rec[valid ? j : lo];
+      const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, bly, blz, chx, bhy, bhz);
+      const bool pass = valid && (BINARY ? (d2 <= rec.w * kCullSlack)
+                                         : (d2 * rec.w <= frm2 * kCullSlack));
+      const unsigned long long m = __ballot(pass);
+      if (m == 0) continue;
+#pragma unroll
+      for (int q = 0; q < kBlocks; ++q) {
+        unsigned mq = (unsigned)(m >> (kPerRound * q)) & ((1u << kPerRound) - 1u);
+        if (mq == 0) continue;
+        // the next record is on its way while this one is evaluated
+        float4 r = s_rec[r0 + __builtin_ctz(mq)];
+        mq &= mq - 1u;                             // loses a bit per trip
+#pragma unroll 1
+        while (true) {
+          const bool more = mq != 0;
+          float4 next = r;
+          if (more) {
+            next = s_rec[r0 + __builtin_ctz(mq)];
+            mq &= mq - 1u;
+          }
+          float val;
+          const bool hit = density_hit<BINARY, false>(g, vx - r.x, vy[q / kBlkPerWave] - r.y,
+                                                      vz[q % kBlkPerWave] - r.z, r.w, 0.f, frm2,
+                                                      grm2, quad_c, val);
+          if (hit) acc[q] = BINARY ? 1.0f : acc[q] + val;
+          if (!more) break;
+          r = next;
+        }
+      }
+    }
+  };
+
+  // ---- common case: one scan, survivors sorted by channel into resident records --------------
+  bool sorted = false;
+  if (natoms <= 65536 && ntypes <= kSortChannels) {
+    const bool one_pass = scan(0, natoms, -1);
+    if (one_pass && ncand <= kRecMax) {
+      sorted = true;
+      for (int i = tid; i < kSegs * kSortChannels; i += kThreads) (&s_cnt[0][0])[i] = 0;
+      __syncthreads();
+      constexpr int kMine = kRecMax / kThreads;   // records per thread
+      float4 rec[kMine];
+      int chan[kMine], rank[kMine];
+#pragma unroll
+      for (int k = 0; k < kMine; ++k) {
+        const int gi = tid + k * kThreads;
+        const bool have = gi < ncand;
+        const int a = have ? atom_of(0, gi) : 0;
+        rec[k] = record_of(a);
+        const float tf = floorf(buffer_float(types_buf, a));
+        const bool act = have && tf >= 0.f && tf < (float)ntypes;   // others feed no channel
+        chan[k] = act ? (int)tf : 0;
+        // lanes of this wave with the same channel
+        unsigned long long same = __ballot(act);
+#pragma unroll
+        for (int bit = 0; bit < 6; ++bit) {
+          const bool set = (chan[k] >> bit) & 1;
+          const unsigned long long bm = __ballot(act && set);
+          same &= set ? bm : ~bm;
+        }
+        rank[k] = act ? __popcll(same & ((1ull << lane) - 1ull)) : -1;
+        if (rank[k] == 0) s_cnt[wave + k * kWaves][chan[k]] = __popcll(same);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        // lane = channel: pieces in order, then channels in order
+        int run = 0;
+#pragma unroll
+        for (int s = 0; s < kSegs; ++s) {
+          const int v = s_cnt[s][lane];
+          s_cnt[s][lane] = run;
+          run += v;
+        }
+        int incl = run;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+          const int t = __shfl_up(incl, d);
+          if (lane >= d) incl += t;
+        }
+        const int excl = incl - run;
+        s_start[lane] = excl;
+        if (lane == kWave - 1) s_start[kWave] = incl;
+#pragma unroll
+        for (int s = 0; s < kSegs; ++s) s_cnt[s][lane] += excl;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < kMine; ++k)
+        if (rank[k] >= 0) s_rec[min(s_cnt[wave + k * kWaves][chan[k]] + rank[k], kRecMax - 1)] = rec[k];
+      __syncthreads();
+    }
+  }
+
+  if (sorted) {
+    for (int c = 0; c < ntypes; ++c) {
+      const int lo = __builtin_amdgcn_readfirstlane(s_start[c]);
+      const int hi = __builtin_amdgcn_readfirstlane(s_start[c + 1]);
+      if (hi > lo) {
+        splat_records(lo, hi);
+        stage_sums();
+        lds_barrier();
+        store_channel(c, true);
+        lds_barrier();
+      } else {
+        store_channel(c, false);
+      }
+    }
+    return;
+  }
+
+  // ---- any size: every channel scans the atoms again, keeping its own -------------------------
+  for (int c = 0; c < ntypes; ++c) {
+    for (int s0 = 0; s0 < natoms; s0 += kSuper) {
+      scan(s0, min(natoms, s0 + kSuper), c);
+      for (int c0 = 0; c0 < ncand; c0 += kRecMax) {
+        const int m = min(kRecMax, ncand - c0);
+        for (int r = tid; r < m; r += kThreads) s_rec[r] = record_of(atom_of(s0, c0 + r));
+        __syncthreads();
+        splat_records(0, m);
+        lds_barrier();
+      }
+    }
+    stage_sums();
+    lds_barrier();
+    store_channel(c, true);
+    lds_barrier();
+  }
+}
+
+}  // namespace
+
+// Returns hipErrorInvalidValue when the kernel does not cover the case (the caller then uses the
+// column kernel): the grids of one example must fit a buffer's 32-bit extent.
+hipError_t launch_forward_channel(const GridArg& g, const BatchArg& batch, int nbatch,
+                                  const Vec3Arg& centers, const float* coords,
+                                  const float* type_index, const float* radii, float* out,
+                                  bool binary, hipStream_t stream) {
+  const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
+  if ((size_t)g.ntypes * chan_stride * 4 >= 0xfffffff0ull) return hipErrorInvalidValue;
+  const int cols_per_side = (g.dim + kColXY - 1) / kColXY;
+  const int slabs = (g.dim + kSlabZ - 1) / kSlabZ;
+  const int aligned = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
+  const int groups = cols_per_side * ((cols_per_side + kCols - 1) / kCols);
+  const dim3 grid(groups * slabs, nbatch), block(kThreads);
+  if (binary)
+    hipLaunchKernelGGL((splat_channel_kernel<true>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, out, cols_per_side, aligned);
+  else
+    hipLaunchKernelGGL((splat_channel_kernel<false>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, out, cols_per_side, aligned);
+  return hipGetLastError();
+}
+
+}  // namespace mg

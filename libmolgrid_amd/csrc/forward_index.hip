@@ -23,6 +23,8 @@
 // Vector types (VEC): every atom feeds all channels, so the splat step multiplies the atom's
 // density into all 28 register sums with the atom's weights, which are read through
 // wave-uniform (scalar) loads; binary mode adds the bare weight, in atom order -> bit exact.
+#include <cstdlib>
+
 #include "kernels.h"
 #include "splat_common.h"
 
@@ -514,6 +516,15 @@ hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nba
                                 const Vec3Arg& centers, const float* coords,
                                 const float* type_index, const float* radii, float* out,
                                 bool binary, bool exact, hipStream_t stream) {
+  static const bool by_channel = [] {
+    const char* v = getenv("MOLGRID_HIP_FORWARD_BY_CHANNEL");
+    return v != nullptr && v[0] == '1';
+  }();
+  if (by_channel && !exact) {
+    const hipError_t e = launch_forward_channel(g, batch, nbatch, centers, coords, type_index,
+                                                radii, out, binary, stream);
+    if (e != hipErrorInvalidValue) return e;
+  }
   return launch_mode<false>(g, batch, nbatch, centers, coords, type_index, radii, out, binary, exact,
                             stream);
 }

@@ -31,6 +31,12 @@ hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nba
                                 const float* type_index, const float* radii, float* out,
                                 bool binary, bool exact, hipStream_t stream);
 
+// index types, one channel at a time (forward_channel.hip); hipErrorInvalidValue = not covered
+hipError_t launch_forward_channel(const GridArg& g, const BatchArg& batch, int nbatch,
+                                  const Vec3Arg& centers, const float* coords,
+                                  const float* type_index, const float* radii, float* out,
+                                  bool binary, hipStream_t stream);
+
 // vector types with per-atom radii: the column kernel of forward_index.hip
 hipError_t launch_forward_vector_column(const GridArg& g, const BatchArg& batch, int nbatch,
                                         const Vec3Arg& centers, const float* coords,
