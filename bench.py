@@ -247,13 +247,13 @@ def main():
 
     dominant_fwd = ms_fwd >= ms_bwd
     roofline = {
-        "kernel": "splat_column_kernel (forward)" if dominant_fwd else "backward_index_kernel",
+        "kernel": "splat_channel_kernel (forward)" if dominant_fwd else "backward_index_kernel",
         "bound": "hbm",
         "achieved": round(fwd_gbs if dominant_fwd else bwd_gbs, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
-        "traffic": measured_traffic("splat_column_kernel" if dominant_fwd
+        "traffic": measured_traffic("splat_channel_kernel" if dominant_fwd
                                     else "backward_index_kernel"),
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),

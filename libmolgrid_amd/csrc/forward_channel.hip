@@ -1,13 +1,14 @@
 // Forward splat for index types, one channel at a time (GridMaker::forward,
 // src/grid_maker.cpp:160-211, src/grid_maker.cu:95-211).
 //
-// A workgroup owns three columns of 4 x 4 voxels in (x, y), consecutive in y, over a slab of up to
-// 48 voxels in z, like the column kernel of forward_index.hip, but walks the channels one after
-// the other: the atoms that can reach the columns are sorted by channel (stably, so each channel
-// keeps ascending atom order), the densities of one channel are summed in nine registers per lane
-// (one voxel in each of the wave's nine 4x4x4 blocks, in atom order), put into an LDS stage that
-// holds the three columns of that channel, and written out as whole z rows.  Only the sums of the
-// current channel live in registers, so the kernel needs few of them and many waves fit a CU.
+// A workgroup owns four columns of 4 x 4 voxels in (x, y), consecutive in y, over a slab of up to
+// 48 voxels in z, one column per wave.  The atoms that can reach the four columns are found by one
+// scan of the example and sorted by channel (stably, so each channel keeps ascending atom order).
+// Each wave then walks the channels on its own: the densities of one channel are summed in twelve
+// registers per lane (one voxel in each of the column's twelve 4x4x4 blocks, in atom order), put
+// into the wave's own LDS stage and written out as whole z rows.  Only the sums of the current
+// channel live in registers, so the kernel needs few of them; after the sort the waves share
+// read-only data only and never wait for each other.
 //
 // Every global access goes through buffer instructions with the extent of the array they address,
 // so an index outside it reads zero or is dropped.
@@ -18,16 +19,13 @@ namespace mg {
 namespace {
 
 constexpr int kColXY = 4;                        // column footprint in x and y
-constexpr int kCols = 3;                         // columns per workgroup
-constexpr int kWaves = 4;
+constexpr int kWaves = 4;                        // = columns per workgroup
 constexpr int kThreads = kWaves * kWave;
-constexpr int kBlkPerWave = 3;                   // 4x4x4 blocks per wave and column
-constexpr int kSlabZ = kWaves * kBlkPerWave * 4; // 48
-constexpr int kBlocks = kCols * kBlkPerWave;     // blocks a wave owns
-constexpr int kPerRound = 7;                     // records per cull round: 7 x 9 blocks = 63 lanes
+constexpr int kBlocks = 12;                      // 4x4x4 blocks of a column
+constexpr int kSlabZ = kBlocks * 4;              // 48
+constexpr int kPerRound = kWave / kBlocks;       // records per cull round: one lane per (record, block)
 constexpr int kRowPad = 52;                      // staged z row, padded against bank conflicts
-constexpr int kPlane = 16 * kRowPad;             // one staged column
-constexpr int kStage = kCols * kPlane;
+constexpr int kPlane = 16 * kRowPad;             // one staged column (floats)
 constexpr int kSuper = 2048;                     // atoms scanned per pass
 constexpr int kSeg = kSuper / kWaves;            // survivors kept per wave
 constexpr int kRecMax = 512;                     // records resident at a time
@@ -35,7 +33,6 @@ constexpr int kSegs = kRecMax / kWave;           // 64-record pieces of the reco
 constexpr int kSortChannels = 64;                // channels the one-pass sort handles
 constexpr int kBufferFlags = 0x00020000;         // untyped 32-bit elements, no swizzle
 
-static_assert(kBlocks * kPerRound <= kWave, "one lane per (record, block) pair of a cull round");
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
@@ -62,7 +59,8 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ types, const float* __restrict__ radii, float* __restrict__ out,
     int cols_per_side, int aligned_rows) {
-  __shared__ __align__(16) float s_stage[kStage];
+  constexpr int kStage = kWaves * kPlane;
+  __shared__ __align__(16) float s_stage[kStage];  // one column per wave
   __shared__ unsigned short s_idx[kWaves][kSeg];
   __shared__ float4 s_rec[kRecMax];                // x, y, z, (ar^2 | 1/ar^2), sorted by channel
   __shared__ int s_wcount[kWaves];
@@ -94,52 +92,50 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
   const __amdgpu_buffer_rsrc_t out_buf =
       buffer_of(out + (size_t)b * ntypes * chan_stride, (size_t)ntypes * chan_stride * 4);
 
-  // which three columns and which z slab
-  const int groups_per_row = (cols_per_side + kCols - 1) / kCols;
+  // which four columns and which z slab
+  const int groups_per_row = (cols_per_side + kWaves - 1) / kWaves;
   const int ngroups = cols_per_side * groups_per_row;
   const int slab = blockIdx.x / ngroups;
   const int grp = blockIdx.x - slab * ngroups;
   const int x0 = (grp / groups_per_row) * kColXY;
-  const int gy0 = (grp % groups_per_row) * (kColXY * kCols);
+  const int gy0 = (grp % groups_per_row) * (kColXY * kWaves);
+  const int y0 = gy0 + wave * kColXY;              // this wave's column
   const int z0 = slab * kSlabZ;
   const int zend = min(z0 + kSlabZ, dim);          // exclusive
+  const bool column_live = y0 < dim;
 
-  // box of the whole group (first/last voxel centre inside the grid)
+  // box of the whole group (first/last voxel centre inside the grid) and of this wave's column
   const float clx = uniform(grid_coord(ox, x0, g.resolution));
   const float chx = uniform(grid_coord(ox, min(x0 + kColXY, dim) - 1, g.resolution));
   const float gly = uniform(grid_coord(oy, gy0, g.resolution));
-  const float ghy = uniform(grid_coord(oy, min(gy0 + kColXY * kCols, dim) - 1, g.resolution));
+  const float ghy = uniform(grid_coord(oy, min(gy0 + kColXY * kWaves, dim) - 1, g.resolution));
   const float clz = uniform(grid_coord(oz, z0, g.resolution));
   const float chz = uniform(grid_coord(oz, zend - 1, g.resolution));
+  const float cly = uniform(grid_coord(oy, min(y0, dim - 1), g.resolution));
+  const float chy = uniform(grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution));
 
-  // the voxels this lane owns: one in each of the wave's nine blocks; a voxel outside the grid
-  // sits at infinity, where no atom reaches it
+  // the voxels this lane owns: one in each of the column's twelve blocks; a voxel outside the
+  // grid sits at infinity, where no atom reaches it
   const int lx = lane >> 4, ly = (lane >> 2) & 3, lz = lane & 3;
-  const int vxi = x0 + lx;
+  const int vxi = x0 + lx, vyi = y0 + ly;
   const float vx = grid_coord(ox, vxi, g.resolution);
-  float vy[kCols], vz[kBlkPerWave];
+  const float vy = grid_coord(oy, vyi, g.resolution);
+  float vz[kBlocks];
 #pragma unroll
-  for (int c = 0; c < kCols; ++c) {
-    const int vyi = gy0 + c * kColXY + ly;
-    vy[c] = (vxi < dim && vyi < dim) ? grid_coord(oy, vyi, g.resolution) : INFINITY;
+  for (int q = 0; q < kBlocks; ++q) {
+    const int vzi = z0 + q * 4 + lz;
+    vz[q] = (vxi < dim && vyi < dim && vzi < zend) ? grid_coord(oz, vzi, g.resolution) : INFINITY;
   }
-#pragma unroll
-  for (int k = 0; k < kBlkPerWave; ++k) {
-    const int vzi = z0 + (wave * kBlkPerWave + k) * 4 + lz;
-    vz[k] = vzi < zend ? grid_coord(oz, vzi, g.resolution) : INFINITY;
-  }
-  const int stage_lane = (lx * 4 + ly) * kRowPad + wave * (kBlkPerWave * 4) + lz;
+  float* const stage = s_stage + wave * kPlane;    // this wave's column
+  const int stage_lane = (lx * 4 + ly) * kRowPad + lz;
 
-  // the (record, block) pair this lane tests in a cull round, and that block's box
-  const int pair_block = lane / kPerRound;         // 0..8; lane 63 tests nothing
+  // the (record, block) pair this lane tests in a cull round, and that block's extent in z
+  const int pair_block = lane / kPerRound;         // lanes past the last block test nothing
   const int pair_rec = lane - pair_block * kPerRound;
-  float bly = INFINITY, bhy = INFINITY, blz = INFINITY, bhz = INFINITY;
-  if (pair_block < kBlocks) {
-    const int y0 = gy0 + (pair_block / kBlkPerWave) * kColXY;
-    const int zb = z0 + (wave * kBlkPerWave + pair_block % kBlkPerWave) * 4;
-    if (y0 < dim && zb < zend && x0 < dim) {
-      bly = grid_coord(oy, y0, g.resolution);
-      bhy = grid_coord(oy, min(y0 + kColXY, dim) - 1, g.resolution);
+  float blz = INFINITY, bhz = INFINITY;
+  if (pair_block < kBlocks && column_live) {
+    const int zb = z0 + pair_block * 4;
+    if (zb < zend) {
       blz = grid_coord(oz, zb, g.resolution);
       bhz = grid_coord(oz, min(zb + 4, zend) - 1, g.resolution);
     }
@@ -151,42 +147,41 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
   const float grm2 = uniform(g.grm * g.grm);
   const float cull_mult = BINARY ? 1.0f : g.frm;   // support radius / ar
 
-  // fixed positions of this thread in the write-out of a channel (float4 granules of z rows)
-  constexpr int kItems = kCols * 16 * (kSlabZ / 4);                 // 576
-  constexpr int kPer = (kItems + kThreads - 1) / kThreads;          // 3
-  int st_lds[kPer], st_off[kPer], st_z[kPer];
+  // this lane's part in the write-out of a channel: three float4 granules; consecutive lanes take
+  // consecutive granules of a z row and the rows follow each other in y, so that one store
+  // instruction of the wave covers up to 1 KiB of contiguous memory
+  constexpr int kPer = (16 * (kSlabZ / 4)) / kWave;                 // 3
+  int st_lds[kPer], st_z[kPer];
+  unsigned st_off[kPer];
 #pragma unroll
   for (int k = 0; k < kPer; ++k) {
-    const int item = tid + k * kThreads;
-    const int col = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
-    const int gx = x0 + (row >> 2), gy = gy0 + col * kColXY + (row & 3), gz = z0 + f4 * 4;
-    st_lds[k] = min(col, kCols - 1) * kPlane + row * kRowPad + f4 * 4;
-    const bool ok = item < kItems && gx < dim && gy < dim && gz < zend;
+    const int item = lane + k * kWave;
+    const int row = item / 12, f4 = item - row * 12;
+    const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
+    st_lds[k] = row * kRowPad + f4 * 4;
+    const bool ok = gx < dim && gy < dim && gz < zend;
     st_z[k] = ok ? gz : dim;                                        // dim: nothing to write
-    st_off[k] = ok ? (int)((unsigned)((gx * dim + gy) * dim + gz) * 4u) : 0;
+    st_off[k] = ok ? (unsigned)((gx * dim + gy) * dim + gz) * 4u : 0u;
   }
 
-  // One channel of the stage (or zeros) -> global memory as z rows.
+  // One channel of the wave's stage (or zeros) -> global memory as z rows.
   auto store_channel = [&](int c, bool from_stage) {
     const unsigned chan_off = (unsigned)c * (unsigned)(chan_stride * 4);   // < 4 GB in total
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
       if (st_z[k] < dim) {
         v4f v = {0.f, 0.f, 0.f, 0.f};
-        if (from_stage) {
-          v = *reinterpret_cast<const v4f*>(s_stage + st_lds[k]);
-        }
+        if (from_stage) v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
+        const unsigned off = chan_off + st_off[k];
         if (aligned_rows && st_z[k] + 3 < dim) {
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf,
-                                                 (int)(chan_off + (unsigned)st_off[k]), 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf, (int)off, 0, 0);
         } else {
           const float e[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
           for (int t = 0; t < 4; ++t)
             if (st_z[k] + t < dim)
-              __builtin_amdgcn_raw_buffer_store_b32(
-                  __builtin_bit_cast(unsigned, e[t]), out_buf,
-                  (int)(chan_off + (unsigned)st_off[k] + 4u * t), 0, 0);
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, e[t]), out_buf,
+                                                    (int)(off + 4u * t), 0, 0);
         }
       }
     }
@@ -262,28 +257,29 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
     return make_float4(ax, ay, az, BINARY ? ar2 : 1.0f / ar2);
   };
 
-  // the sums of the current channel at this lane's nine voxels
+  // the sums of the current channel at this lane's twelve voxels
   float acc[kBlocks];
 #pragma unroll
   for (int q = 0; q < kBlocks; ++q) acc[q] = 0.f;
-  // sums -> stage (cleared for the next channel); the caller synchronises
+  // sums -> the wave's stage (and cleared for the next channel); the wave reads them back itself,
+  // and LDS keeps the order of one wave's accesses
   auto stage_sums = [&]() {
 #pragma unroll
     for (int q = 0; q < kBlocks; ++q) {
-      s_stage[stage_lane + (q / kBlkPerWave) * kPlane + (q % kBlkPerWave) * 4] = acc[q];
+      stage[stage_lane + q * 4] = acc[q];
       acc[q] = 0.f;
     }
   };
 
   // ---- records [lo, hi) of s_rec, all of one channel, added to the sums -----------------------
-  // A cull round tests seven records against the wave's nine blocks, one pair per lane; the pairs
-  // that pass are taken block by block and, within a block, in record order.
+  // A cull round tests five records against the column's twelve blocks, one pair per lane; the
+  // pairs that pass are taken block by block and, within a block, in record order.
   auto splat_records = [&](int lo, int hi) {
     for (int r0 = lo; r0 < hi; r0 += kPerRound) {
       const int j = r0 + pair_rec;
       const bool valid = pair_block < kBlocks && j < hi;
       const float4 rec = s_rec[valid ? j : lo];
-      const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, bly, blz, chx, bhy, bhz);
+      const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
       const bool pass = valid && (BINARY ? (d2 <= rec.w * kCullSlack)
                                          : (d2 * rec.w <= frm2 * kCullSlack));
       const unsigned long long m = __ballot(pass);
@@ -291,25 +287,33 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
 #pragma unroll
       for (int q = 0; q < kBlocks; ++q) {
         unsigned mq = (unsigned)(m >> (kPerRound * q)) & ((1u << kPerRound) - 1u);
-        if (mq == 0) continue;
-        // the next record is on its way while this one is evaluated
-        float4 r = s_rec[r0 + __builtin_ctz(mq)];
-        mq &= mq - 1u;                             // loses a bit per trip
+        // the record of a passing pair comes straight from the lane that tested it
 #pragma unroll 1
-        while (true) {
-          const bool more = mq != 0;
-          float4 next = r;
-          if (more) {
-            next = s_rec[r0 + __builtin_ctz(mq)];
-            mq &= mq - 1u;
+        while (mq != 0) {                          // loses a bit per trip
+          const int src = q * kPerRound + __builtin_ctz(mq);
+          mq &= mq - 1u;
+          const float rx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.x), src));
+          const float ry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.y), src));
+          const float rz = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.z), src));
+          const float rw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.w), src));
+          const float dx = vx - rx, dy = vy - ry, dz = vz[q] - rz;
+          if (BINARY) {
+            if (sq_distance_exact(dx, dy, dz) < rw) acc[q] = 1.0f;
+          } else {
+            // the density of splat_common.h's density_hit; the exponential is evaluated only when
+            // some voxel of the block lies inside the atom's Gaussian core
+            const float u = (dx * dx + dy * dy + dz * dz) * rw;
+            if (u <= frm2) {
+              const float su = __builtin_amdgcn_sqrtf(u);
+              float val = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+              const bool core = u <= grm2;
+              if (__ballot(core) != 0) {
+                const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                val = core ? gauss : val;
+              }
+              acc[q] += val;
+            }
           }
-          float val;
-          const bool hit = density_hit<BINARY, false>(g, vx - r.x, vy[q / kBlkPerWave] - r.y,
-                                                      vz[q % kBlkPerWave] - r.z, r.w, 0.f, frm2,
-                                                      grm2, quad_c, val);
-          if (hit) acc[q] = BINARY ? 1.0f : acc[q] + val;
-          if (!more) break;
-          r = next;
         }
       }
     }
@@ -377,15 +381,14 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
   }
 
   if (sorted) {
+    if (!column_live) return;
     for (int c = 0; c < ntypes; ++c) {
       const int lo = __builtin_amdgcn_readfirstlane(s_start[c]);
       const int hi = __builtin_amdgcn_readfirstlane(s_start[c + 1]);
       if (hi > lo) {
         splat_records(lo, hi);
         stage_sums();
-        lds_barrier();
         store_channel(c, true);
-        lds_barrier();
       } else {
         store_channel(c, false);
       }
@@ -401,14 +404,14 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
         const int m = min(kRecMax, ncand - c0);
         for (int r = tid; r < m; r += kThreads) s_rec[r] = record_of(atom_of(s0, c0 + r));
         __syncthreads();
-        splat_records(0, m);
-        lds_barrier();
+        if (column_live) splat_records(0, m);
+        lds_barrier();   // before the records are built again
       }
     }
-    stage_sums();
-    lds_barrier();
-    store_channel(c, true);
-    lds_barrier();
+    if (column_live) {
+      stage_sums();
+      store_channel(c, true);
+    }
   }
 }
 
@@ -425,7 +428,7 @@ hipError_t launch_forward_channel(const GridArg& g, const BatchArg& batch, int n
   const int cols_per_side = (g.dim + kColXY - 1) / kColXY;
   const int slabs = (g.dim + kSlabZ - 1) / kSlabZ;
   const int aligned = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
-  const int groups = cols_per_side * ((cols_per_side + kCols - 1) / kCols);
+  const int groups = cols_per_side * ((cols_per_side + kWaves - 1) / kWaves);
   const dim3 grid(groups * slabs, nbatch), block(kThreads);
   if (binary)
     hipLaunchKernelGGL((splat_channel_kernel<true>), grid, block, 0, stream, g, batch, centers,

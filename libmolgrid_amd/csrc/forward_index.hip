@@ -516,11 +516,11 @@ hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nba
                                 const Vec3Arg& centers, const float* coords,
                                 const float* type_index, const float* radii, float* out,
                                 bool binary, bool exact, hipStream_t stream) {
-  static const bool by_channel = [] {
-    const char* v = getenv("MOLGRID_HIP_FORWARD_BY_CHANNEL");
-    return v != nullptr && v[0] == '1';
-  }();
-  if (by_channel && !exact) {
+  // The channel-by-channel kernel takes every case it covers (anything but the exact cut-off
+  // predicates and grids of 4 GB or more per example); MOLGRID_HIP_FORWARD_COLUMN_KERNEL=1 keeps
+  // the column kernel below for all of them (a tested second implementation).
+  const char* column_only = getenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL");
+  if (!exact && !(column_only != nullptr && column_only[0] == '1')) {
     const hipError_t e = launch_forward_channel(g, batch, nbatch, centers, coords, type_index,
                                                 radii, out, binary, stream);
     if (e != hipErrorInvalidValue) return e;

@@ -188,3 +188,35 @@ def test_repeat_runs_are_bit_identical(mg):
     gm.forward_batch(*args, a)
     gm.forward_batch(*args, b)
     assert torch.equal(a, b)
+
+
+def test_more_channels_than_the_channel_sort_handles(mg):
+    """70 channels: every channel scans the atoms again instead of one sort (any channel count)."""
+    rng = np.random.default_rng(70)
+    coords, types, radii = synth.small_index_case(rng, 400, 70, 8.0)
+    for binary in (False, True):
+        ref = oracle.GridMaker(0.5, 11.5, binary).forward((0, 0, 0), coords, types, radii, 70)
+        got = gpu_forward(mg, (0.5, 11.5, binary), (0, 0, 0), coords, types, radii, 70)
+        if binary:
+            assert np.array_equal(got, ref)
+        else:
+            assert_close(got, ref, what="70 channels")
+
+
+def test_column_kernel_gives_the_same_values(mg, monkeypatch):
+    """The second implementation of the index-type forward pass (one column of all channels per
+    pass) sums in the same order: identical grids, dense and binary, also for a ragged batch."""
+    rng = np.random.default_rng(5)
+    coords, types, radii = synth.small_index_case(rng, 900, 28, 14.0)
+    for binary in (False, True):
+        monkeypatch.delenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL", raising=False)
+        a = gpu_forward(mg, (0.5, 23.5, binary), (0.3, -0.2, 0.1), coords, types, radii, 28)
+        monkeypatch.setenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL", "1")
+        b = gpu_forward(mg, (0.5, 23.5, binary), (0.3, -0.2, 0.1), coords, types, radii, 28)
+        monkeypatch.delenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL")
+        assert np.array_equal(a, b)
+        ref = oracle.GridMaker(0.5, 23.5, binary).forward((0.3, -0.2, 0.1), coords, types, radii, 28)
+        if binary:
+            assert np.array_equal(b, ref)
+        else:
+            assert_close(b, ref, what="column kernel")
