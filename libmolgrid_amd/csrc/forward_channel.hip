@@ -54,21 +54,26 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Seven workgroups per CU (72 registers): the launch of configuration 1 (1,800 workgroups) then
+// fits the 1,792 slots of the chip in one go.
 template <bool BINARY>
-__global__ __launch_bounds__(kThreads) void splat_channel_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(7, 7))) void
+splat_channel_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ types, const float* __restrict__ radii, float* __restrict__ out,
     int cols_per_side, int aligned_rows) {
   constexpr int kStage = kWaves * kPlane;
   __shared__ __align__(16) float s_stage[kStage];  // one column per wave
-  __shared__ unsigned short s_idx[kWaves][kSeg];
   __shared__ float4 s_rec[kRecMax];                // x, y, z, (ar^2 | 1/ar^2), sorted by channel
   __shared__ int s_wcount[kWaves];
   __shared__ int s_start[kSortChannels + 1];       // first record of each channel
 
-  // records per (64-record piece, channel) while the records are sorted: the stage is not in use then
-  int (*s_cnt)[kSortChannels] = reinterpret_cast<int (*)[kSortChannels]>(s_stage);
-  static_assert(kSegs * kSortChannels <= kStage, "the counts fit the stage");
+  // The stage is not in use while atoms are scanned and sorted; it then holds the survivors of
+  // the scan (atom numbers) and the records per (64-record piece, channel).
+  unsigned short (*s_idx)[kSeg] = reinterpret_cast<unsigned short (*)[kSeg]>(s_stage);
+  int (*s_cnt)[kSortChannels] =
+      reinterpret_cast<int (*)[kSortChannels]>(s_stage + kWaves * kSeg / 2);
+  static_assert(kWaves * kSeg / 2 + kSegs * kSortChannels <= kStage, "both fit the stage");
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -147,39 +152,32 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
   const float grm2 = uniform(g.grm * g.grm);
   const float cull_mult = BINARY ? 1.0f : g.frm;   // support radius / ar
 
-  // this lane's part in the write-out of a channel: three float4 granules; consecutive lanes take
-  // consecutive granules of a z row and the rows follow each other in y, so that one store
-  // instruction of the wave covers up to 1 KiB of contiguous memory
-  constexpr int kPer = (16 * (kSlabZ / 4)) / kWave;                 // 3
-  int st_lds[kPer], st_z[kPer];
-  unsigned st_off[kPer];
-#pragma unroll
-  for (int k = 0; k < kPer; ++k) {
-    const int item = lane + k * kWave;
-    const int row = item / 12, f4 = item - row * 12;
-    const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
-    st_lds[k] = row * kRowPad + f4 * 4;
-    const bool ok = gx < dim && gy < dim && gz < zend;
-    st_z[k] = ok ? gz : dim;                                        // dim: nothing to write
-    st_off[k] = ok ? (unsigned)((gx * dim + gy) * dim + gz) * 4u : 0u;
-  }
+  // this lane's part in the write-out of a channel: for each of the column's four x, lane
+  // (y, granule) takes one float4 piece of a z row; the four rows of an x follow each other in
+  // memory, so one store instruction of the wave covers 768 contiguous bytes
+  const int st_y = lane / 12, st_f4 = lane - st_y * 12;           // lanes 48..63 idle
+  const int st_gz = z0 + st_f4 * 4;
+  const bool st_lane_live = st_y < 4 && y0 + st_y < dim && st_gz < zend;
+  const int st_lds = st_y * kRowPad + st_f4 * 4;
+  const unsigned st_off = (unsigned)((x0 * dim + y0 + st_y) * dim + st_gz) * 4u;
+  const unsigned st_xstride = (unsigned)(dim * dim) * 4u;
 
   // One channel of the wave's stage (or zeros) -> global memory as z rows.
   auto store_channel = [&](int c, bool from_stage) {
     const unsigned chan_off = (unsigned)c * (unsigned)(chan_stride * 4);   // < 4 GB in total
 #pragma unroll
-    for (int k = 0; k < kPer; ++k) {
-      if (st_z[k] < dim) {
+    for (int k = 0; k < kColXY; ++k) {
+      if (st_lane_live && x0 + k < dim) {
         v4f v = {0.f, 0.f, 0.f, 0.f};
-        if (from_stage) v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
-        const unsigned off = chan_off + st_off[k];
-        if (aligned_rows && st_z[k] + 3 < dim) {
+        if (from_stage) v = *reinterpret_cast<const v4f*>(stage + st_lds + k * 4 * kRowPad);
+        const unsigned off = chan_off + st_off + k * st_xstride;
+        if (aligned_rows && st_gz + 3 < dim) {
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf, (int)off, 0, 0);
         } else {
           const float e[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (st_z[k] + t < dim)
+            if (st_gz + t < dim)
               __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, e[t]), out_buf,
                                                     (int)(off + 4u * t), 0, 0);
         }
@@ -296,24 +294,10 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
           const float ry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.y), src));
           const float rz = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.z), src));
           const float rw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.w), src));
-          const float dx = vx - rx, dy = vy - ry, dz = vz[q] - rz;
-          if (BINARY) {
-            if (sq_distance_exact(dx, dy, dz) < rw) acc[q] = 1.0f;
-          } else {
-            // the density of splat_common.h's density_hit; the exponential is evaluated only when
-            // some voxel of the block lies inside the atom's Gaussian core
-            const float u = (dx * dx + dy * dy + dz * dz) * rw;
-            if (u <= frm2) {
-              const float su = __builtin_amdgcn_sqrtf(u);
-              float val = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
-              const bool core = u <= grm2;
-              if (__ballot(core) != 0) {
-                const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
-                val = core ? gauss : val;
-              }
-              acc[q] += val;
-            }
-          }
+          float val;
+          const bool hit = density_hit<BINARY, false>(g, vx - rx, vy - ry, vz[q] - rz, rw, 0.f, frm2,
+                                                      grm2, quad_c, val);
+          if (hit) acc[q] = BINARY ? 1.0f : acc[q] + val;
         }
       }
     }
@@ -382,7 +366,12 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
 
   if (sorted) {
     if (!column_live) return;
-    for (int c = 0; c < ntypes; ++c) {
+    // Channels differ a lot in work (some hold most atoms, many hold none, and an empty channel is
+    // stores only), so the waves start at different channels: at any time some compute while
+    // others store.  The order of the channels does not matter to the sums.
+    const int first = (int)((blockIdx.x * 7u + blockIdx.y * 3u + wave * 5u) % (unsigned)ntypes);
+    for (int i = 0; i < ntypes; ++i) {
+      const int c = first + i < ntypes ? first + i : first + i - ntypes;
       const int lo = __builtin_amdgcn_readfirstlane(s_start[c]);
       const int hi = __builtin_amdgcn_readfirstlane(s_start[c + 1]);
       if (hi > lo) {
@@ -412,6 +401,7 @@ __global__ __launch_bounds__(kThreads) void splat_channel_kernel(
       stage_sums();
       store_channel(c, true);
     }
+    lds_barrier();   // the stage holds the next scan's survivors
   }
 }
 
