@@ -55,6 +55,8 @@ def test_density_profile_closed_form(mg):
     (0.25, 5.75, 2, 15),    # dim 24
     (1.0, 15.0, 40, 200),   # dim 16, more channels than one LDS pass holds
     (0.5, 23.5, 28, 300),   # dim 48
+    (0.5, 29.5, 4, 500),    # dim 60: two slabs in z, the second one partial
+    (0.25, 25.25, 3, 400),  # dim 102: three slabs, rows that are not a multiple of four voxels
 ])
 @pytest.mark.parametrize("binary", [False, True])
 def test_small_random_vs_oracle(mg, res, dimension, ntypes, natoms, binary):
