@@ -9,6 +9,8 @@
 // loop does (src/grid_maker.cpp:226-270), so binary mode (`+= weight`) is
 // reproduced bit for bit.  The tile is staged through LDS and streamed out as
 // float4 rows.
+#include <cstdlib>
+
 #include "kernels.h"
 #include "splat_common.h"
 
@@ -263,6 +265,12 @@ hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nb
                                  hipStream_t stream) {
   // per-atom radii take the column kernel; type-indexed radii and the exact-predicate modes
   // (truncated Gaussian) use the cubic-tile kernel below
+  // (densities: the matrix-core kernel; MOLGRID_HIP_VECTOR_COLUMN_KERNEL=1 keeps the column kernel,
+  // which binary occupancy always uses because its sums are compared bit for bit)
+  const char* column_only = getenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL");
+  if (!radii_type_indexed && !exact && !binary && !(column_only != nullptr && column_only[0] == '1'))
+    return launch_forward_vector_mfma(g, batch, nbatch, centers, coords, type_vector, radii, out,
+                                      stream);
   if (!radii_type_indexed && !exact)
     return launch_forward_vector_column(g, batch, nbatch, centers, coords, type_vector, radii, out,
                                         binary, exact, stream);

@@ -43,6 +43,12 @@ hipError_t launch_forward_vector_column(const GridArg& g, const BatchArg& batch,
                                         const float* type_vector, const float* radii, float* out,
                                         bool binary, bool exact, hipStream_t stream);
 
+// vector types with per-atom radii, density mode, on the matrix cores (forward_vector_mfma.hip)
+hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
+                                      const Vec3Arg& centers, const float* coords,
+                                      const float* type_vector, const float* radii, float* out,
+                                      hipStream_t stream);
+
 hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
                                  const Vec3Arg& centers, const float* coords,
                                  const float* type_vector, const float* radii, float* out,
