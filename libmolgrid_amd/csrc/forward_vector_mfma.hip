@@ -59,9 +59,9 @@ splat_vector_mfma_kernel(
   __shared__ int s_wcount[kColWaves];
   __shared__ float4 s_rec[kRecChunk];            // x, y, z, 1/ar^2
   __shared__ int s_recatom[kRecChunk];
-  // wave-private list of a block's atoms, four per entry; two spare entries because the loop
-  // reads ahead
-  __shared__ __align__(16) unsigned char s_mini[kColWaves][(kWave / 4 + 2) * kEntryBytes];
+  // wave-private list of a block's atoms, four per entry; spare entries because the loop reads
+  // ahead
+  __shared__ __align__(16) unsigned char s_mini[kColWaves][(kWave / 4 + 3) * kEntryBytes];
   __shared__ __align__(16) float s_stage[2 * kStageCh * kPlane];
 
   const int tid = threadIdx.x;
@@ -246,6 +246,9 @@ splat_vector_mfma_kernel(
                 s.r = *reinterpret_cast<const float4*>(e + quad * 16);
                 const int atom = *reinterpret_cast<const int*>(e + 64 + quad * 4);
                 const bool have = 4 * k + quad < n;   // (past the list: an older atom, unused)
+                // a slot past the list holds anything: no reach at all, so its density is zero
+                // (zero weight alone would not do: 0 * inf is not a number)
+                s.r.w = have ? s.r.w : INFINITY;
                 const float* __restrict__ wa = weights + (size_t)atom * ntypes;
                 s.w0 = (have && chan_live[0]) ? wa[0] : 0.f;
                 s.w1 = (have && chan_live[1]) ? wa[16] : 0.f;
@@ -254,7 +257,7 @@ splat_vector_mfma_kernel(
               const int steps = (n + 3) >> 2;
               Step cur = fetch(0);
               for (int k = 0; k < steps; ++k) {
-                const Step nxt = fetch(k + 1);
+                const Step nxt = fetch(k + 1);   // in flight while this entry is evaluated
                 const float dy = vy - cur.r.y, dz = vz - cur.r.z;
                 const float dyz2 = dy * dy + dz * dz;
 #pragma unroll

@@ -106,6 +106,28 @@ def test_config3_shape_vs_oracle(mg, binary):
         assert_close(out.cpu().numpy(), ref, what="config 3")
 
 
+def test_column_kernel_agrees_with_the_matrix_core_kernel(mg, monkeypatch):
+    """Densities of vector-typed atoms: the column kernel (sums in atom order) and the matrix-core
+    kernel (four atoms per multiply-accumulate step) agree to rounding, and both with the oracle;
+    a dense case, more than 32 channels and a grid with partial columns."""
+    rng = np.random.default_rng(8)
+    for natoms, ntypes, gm_args in ((2500, 28, (0.5, 11.5)), (300, 37, (0.5, 6.0))):
+        coords, tv, radii = make_case(rng, natoms, ntypes, gm_args[1] / 2 + 1.0)
+        gm = mg.GridMaker(*gm_args)
+        shape = gm.grid_dimensions(ntypes)
+        monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", raising=False)
+        a = torch.full(shape, 7.0, device="cuda")
+        gm.forward((0, 0, 0), dev(coords), dev(tv), dev(radii), a)
+        monkeypatch.setenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", "1")
+        b = torch.full(shape, 7.0, device="cuda")
+        gm.forward((0, 0, 0), dev(coords), dev(tv), dev(radii), b)
+        monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
+        ref = oracle.GridMaker(*gm_args).forward((0, 0, 0), coords, tv, radii)
+        assert_close(a.cpu().numpy(), ref, rtol=2e-5, what="matrix-core kernel")
+        assert_close(b.cpu().numpy(), ref, rtol=2e-5, what="column kernel")
+        assert not np.isnan(a.cpu().numpy()).any()
+
+
 @pytest.mark.parametrize("ntypes,binary,rti", [(3, False, False), (28, False, False),
                                                (37, False, False), (5, True, False),
                                                (6, False, True), (6, True, True)])
