@@ -222,3 +222,18 @@ def test_column_kernel_gives_the_same_values(mg, monkeypatch):
             assert np.array_equal(b, ref)
         else:
             assert_close(b, ref, what="column kernel")
+
+
+def test_more_atoms_than_sixteen_bit_indices(mg):
+    """70,000 atoms in one example (survivor lists hold 16-bit atom numbers: the atoms are then
+    taken in passes), most of them far from the grid; dense and binary."""
+    rng = np.random.default_rng(77)
+    coords, types, radii = synth.small_index_case(rng, 70000, 4, 30.0)
+    for binary in (False, True):
+        ref = oracle.GridMaker(0.5, 11.5, binary).forward((1.0, -2.0, 0.5), coords, types, radii, 4)
+        got = gpu_forward(mg, (0.5, 11.5, binary), (1.0, -2.0, 0.5), coords, types, radii, 4)
+        if binary:
+            assert np.array_equal(got, ref)
+        else:
+            assert_close(got, ref, what="70,000 atoms")
+    assert ref.sum() > 100
