@@ -184,9 +184,11 @@ splat_vector_mfma_kernel(
 
   for (int cbase = 0; cbase < ntypes; cbase += kChannels) {
     const int nchan = min(kChannels, ntypes - cbase);
-    // this lane's two rows of the weight matrix: channels cbase + j and cbase + 16 + j of every atom
-    const float* __restrict__ weights = type_vector + cbase + j;
+    // this lane's two rows of the weight matrix: channels cbase + j and cbase + 16 + j of every
+    // atom (a row past the last channel reads the last channel and is zeroed afterwards)
     const bool chan_live[2] = {j < nchan, 16 + j < nchan};
+    const float* __restrict__ weights0 = type_vector + cbase + min(j, nchan - 1);
+    const float* __restrict__ weights1 = type_vector + cbase + min(16 + j, nchan - 1);
     for (int col = 0; col < kColsPerGroup; ++col) {
       const int y0 = gy0 + col * kColXY;
       if (y0 >= dim) break;
@@ -239,38 +241,45 @@ splat_vector_mfma_kernel(
               // one entry = four atoms = one step of the matrix product; the quarter wave that
               // holds atom `quad` reads its record and its two weights, every lane evaluates four
               // densities (its (y, z) in each of the four x planes)
-              struct Step { float4 r; float w0, w1; };
+              struct Step { float4 r; float w0, w1; bool have; };
               auto fetch = [&](int k) -> Step {
                 const unsigned char* e = mine + k * kEntryBytes;
                 Step s;
                 s.r = *reinterpret_cast<const float4*>(e + quad * 16);
                 const int atom = *reinterpret_cast<const int*>(e + 64 + quad * 4);
-                const bool have = 4 * k + quad < n;   // (past the list: an older atom, unused)
-                // a slot past the list holds anything: no reach at all, so its density is zero
-                // (zero weight alone would not do: 0 * inf is not a number)
-                s.r.w = have ? s.r.w : INFINITY;
-                const float* __restrict__ wa = weights + (size_t)atom * ntypes;
-                s.w0 = (have && chan_live[0]) ? wa[0] : 0.f;
-                s.w1 = (have && chan_live[1]) ? wa[16] : 0.f;
+                s.have = 4 * k + quad < n;   // (past the list: an older atom or none)
+                // Both weights are always loaded (from the example's first atom where there is
+                // none) and masked only when they are used, an iteration later: the loads of
+                // the next entry then stay in flight while this entry is evaluated.
+                const size_t row = (size_t)(s.have ? atom : begin) * ntypes;
+                s.w0 = weights0[row];
+                s.w1 = weights1[row];
                 return s;
               };
               const int steps = (n + 3) >> 2;
               Step cur = fetch(0);
               for (int k = 0; k < steps; ++k) {
                 const Step nxt = fetch(k + 1);   // in flight while this entry is evaluated
+                __builtin_amdgcn_sched_barrier(0);  // (keeps the loads up here)
+                // a slot past the list has no reach at all, so its density is exactly zero (zero
+                // weight alone would not do: a stale record can give an infinite density, and
+                // 0 * inf is not a number)
+                const float rw = cur.have ? cur.r.w : INFINITY;
+                const float w0 = (cur.have && chan_live[0]) ? cur.w0 : 0.f;
+                const float w1 = (cur.have && chan_live[1]) ? cur.w1 : 0.f;
                 const float dy = vy - cur.r.y, dz = vz - cur.r.z;
                 const float dyz2 = dy * dy + dz * dz;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                   const float dx = vx[t] - cur.r.x;
-                  const float u = (dx * dx + dyz2) * cur.r.w;
+                  const float u = (dx * dx + dyz2) * rw;
                   const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
                   const float su = __builtin_amdgcn_sqrtf(u);
                   const float quadr = fmaxf(fmaf(g.A, u, fmaf(g.B, su, g.C)), 0.f);
                   float d = (u <= grm2) ? gauss : quadr;
                   d = (u <= frm2) ? d : 0.f;
-                  sums[blk][t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.w0, d, sums[blk][t][0], 0, 0, 0);
-                  sums[blk][t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.w1, d, sums[blk][t][1], 0, 0, 0);
+                  sums[blk][t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w0, d, sums[blk][t][0], 0, 0, 0);
+                  sums[blk][t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w1, d, sums[blk][t][1], 0, 0, 0);
                 }
                 cur = nxt;
               }
