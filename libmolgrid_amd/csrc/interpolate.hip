@@ -344,31 +344,86 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   // Two register sets, so that the loads of a channel are issued a whole channel before they are
   // needed: while channel ch is interpolated from one buffer, channel ch + 1 is written to the
-  // other and channel ch + 2 is in flight.
+  // other and channel ch + 2 is in flight.  Every load and store of the loop is issued
+  // unconditionally -- unused staging slots read element 0 into a spare LDS cell, voxels outside
+  // the output grid store through a buffer descriptor to an offset past its end, which the
+  // hardware drops -- because loads and stores share one in-order counter: only with a fixed
+  // number of them per iteration can a wait for channel ch + 1 leave the loads of channel ch + 2
+  // and the stores of channel ch in flight.
   float ra[kFewRounds], rb[kFewRounds];
   auto fetch = [&](float (&r)[kFewRounds], int ch) {
+    const float* chan = src + (size_t)ch * in_chan;
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e) r[e] = chan[st_src[e]];
+  };
+  auto deposit = [&](const float (&r)[kFewRounds], int ch) {
+    const int base = (ch & 1) * kWinSize;
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e)   // (the spare slot is the same for both buffers)
+      s_win[st_dst[e] == 2 * kWinSize ? 2 * kWinSize : base + st_dst[e]] = r[e];
+  };
+  const size_t out_bytes = (size_t)C * out_points * sizeof(float);
+  if (out_bytes < 0x7fffffffull) {
+    const __amdgpu_buffer_rsrc_t out_buf = __builtin_amdgcn_make_buffer_rsrc(
+        out + (size_t)b * C * out_points, 0, (int)out_bytes, 0x00020000);
+    unsigned off[kVox];
+#pragma unroll
+    for (int v = 0; v < kVox; ++v)
+      off[v] = live[v] ? (unsigned)((((size_t)i0 * od + j) * od + k + v * vox_step) * sizeof(float))
+                       : (unsigned)out_bytes;            // past the end for every channel
+    auto interpolate_buffered = [&](int ch, int which) {
+      const float* buf = s_win + which * kWinSize;
+      const unsigned chan_off = (unsigned)((size_t)ch * out_points * sizeof(float));
+#pragma unroll
+      for (int v = 0; v < kVox; ++v) {
+        const float* w = buf + tap[v];
+        float val = w[0] * cw[v][0];
+        val = fmaf(w[1], cw[v][1], val);
+        val = fmaf(w[kWinZ], cw[v][2], val);
+        val = fmaf(w[kWinZ + 1], cw[v][3], val);
+        val = fmaf(w[kWin * kWinZ], cw[v][4], val);
+        val = fmaf(w[kWin * kWinZ + 1], cw[v][5], val);
+        val = fmaf(w[kWin * kWinZ + kWinZ], cw[v][6], val);
+        val = fmaf(w[kWin * kWinZ + kWinZ + 1], cw[v][7], val);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), out_buf,
+                                              (int)(off[v] + chan_off), 0, 0);
+      }
+    };
+    fetch(ra, 0);
+    deposit(ra, 0);
+    fetch(ra, C > 1 ? 1 : 0);
+    __syncthreads();
+    for (int ch = 0; ch < C; ch += 2) {
+      fetch(rb, ch + 2 < C ? ch + 2 : ch);
+      if (ch + 1 < C) deposit(ra, ch + 1);
+      interpolate_buffered(ch, 0);
+      __syncthreads();
+      if (ch + 1 >= C) break;
+      fetch(ra, ch + 3 < C ? ch + 3 : ch);
+      if (ch + 2 < C) deposit(rb, ch + 2);
+      interpolate_buffered(ch + 1, 1);
+      __syncthreads();
+    }
+    return;
+  }
+  // grids of 2 GB or more per example: plain stores under their conditions
+  auto fetch_some = [&](float (&r)[kFewRounds], int ch) {
     const float* chan = src + (size_t)ch * in_chan;
 #pragma unroll
     for (int e = 0; e < kFewRounds; ++e)
       if (e < rounds_used) r[e] = chan[st_src[e]];
   };
-  auto deposit = [&](const float (&r)[kFewRounds], int ch) {
-    float* win = s_win + (ch & 1) * kWinSize;
-#pragma unroll
-    for (int e = 0; e < kFewRounds; ++e)
-      if (e < rounds_used) win[st_dst[e]] = r[e];
-  };
-  fetch(ra, 0);
+  fetch_some(ra, 0);
   deposit(ra, 0);
-  if (C > 1) fetch(ra, 1);
+  if (C > 1) fetch_some(ra, 1);
   __syncthreads();
   for (int ch = 0; ch < C; ch += 2) {
-    if (ch + 2 < C) fetch(rb, ch + 2);
+    if (ch + 2 < C) fetch_some(rb, ch + 2);
     if (ch + 1 < C) deposit(ra, ch + 1);
     interpolate_channel(ch, 0);
     __syncthreads();
     if (ch + 1 >= C) break;
-    if (ch + 3 < C) fetch(ra, ch + 3);
+    if (ch + 3 < C) fetch_some(ra, ch + 3);
     if (ch + 2 < C) deposit(rb, ch + 2);
     interpolate_channel(ch + 1, 1);
     __syncthreads();
