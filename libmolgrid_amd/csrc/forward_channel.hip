@@ -23,7 +23,6 @@ constexpr int kWaves = 4;                        // = columns per workgroup
 constexpr int kThreads = kWaves * kWave;
 constexpr int kBlocks = 12;                      // 4x4x4 blocks of a column
 constexpr int kSlabZ = kBlocks * 4;              // 48
-constexpr int kPerRound = kWave / kBlocks;       // records per cull round: one lane per (record, block)
 constexpr int kRowPad = 52;                      // staged z row, padded against bank conflicts
 constexpr int kPlane = 16 * kRowPad;             // one staged column (floats)
 constexpr int kSuper = 2048;                     // atoms scanned per pass
@@ -133,18 +132,6 @@ splat_channel_kernel(
   }
   float* const stage = s_stage + wave * kPlane;    // this wave's column
   const int stage_lane = (lx * 4 + ly) * kRowPad + lz;
-
-  // the (record, block) pair this lane tests in a cull round, and that block's extent in z
-  const int pair_block = lane / kPerRound;         // lanes past the last block test nothing
-  const int pair_rec = lane - pair_block * kPerRound;
-  float blz = INFINITY, bhz = INFINITY;
-  if (pair_block < kBlocks && column_live) {
-    const int zb = z0 + pair_block * 4;
-    if (zb < zend) {
-      blz = grid_coord(oz, zb, g.resolution);
-      bhz = grid_coord(oz, min(zb + 4, zend) - 1, g.resolution);
-    }
-  }
 
   float quad_c = g.C;
   asm volatile("" : "+v"(quad_c));          // vector register (an fma takes one scalar operand)
@@ -270,26 +257,40 @@ splat_channel_kernel(
   };
 
   // ---- records [lo, hi) of s_rec, all of one channel, added to the sums -----------------------
-  // A cull round tests five records against the column's twelve blocks, one pair per lane; the
-  // pairs that pass are taken block by block and, within a block, in record order.
+  // A cull round takes 64 records, one per lane: the lane finds the interval of z the atom can
+  // reach inside the column (its reach shrunk by the distance to the column's footprint in x and
+  // y) and from it the range of blocks, as a bit mask.  One ballot per block then gives the
+  // records of that block, which are taken in record order; the atom's record comes straight from
+  // the lane that tested it.
+  const float inv_block = 0.25f / g.resolution;             // blocks per unit length along z
+  const int last_block = (zend - z0 + 3) / 4 - 1;
   auto splat_records = [&](int lo, int hi) {
-    for (int r0 = lo; r0 < hi; r0 += kPerRound) {
-      const int j = r0 + pair_rec;
-      const bool valid = pair_block < kBlocks && j < hi;
-      const float4 rec = s_rec[valid ? j : lo];
-      const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
-      const bool pass = valid && (BINARY ? (d2 <= rec.w * kCullSlack)
-                                         : (d2 * rec.w <= frm2 * kCullSlack));
-      const unsigned long long m = __ballot(pass);
-      if (m == 0) continue;
+    for (int r0 = lo; r0 < hi; r0 += kWave) {
+      const int i = r0 + lane;
+      const bool valid = i < hi;
+      const float4 rec = s_rec[valid ? i : lo];
+      const float ex = fmaxf(fmaxf(clx - rec.x, rec.x - chx), 0.f);
+      const float ey = fmaxf(fmaxf(cly - rec.y, rec.y - chy), 0.f);
+      // squared reach (with the slack that keeps the cull a superset) minus the part spent in x, y
+      const float reach2 = (BINARY ? rec.w : frm2 * __builtin_amdgcn_rcpf(rec.w)) * kCullSlack;
+      const float rz2 = reach2 - (ex * ex + ey * ey);
+      unsigned blocks = 0;
+      if (valid && rz2 >= 0.f) {
+        const float rz = __builtin_amdgcn_sqrtf(rz2);
+        // block q holds the voxel centres clz + (4q .. 4q+3) * resolution
+        const float top = (rec.z + rz - clz) * inv_block + 1e-3f;
+        const float bottom = (rec.z - rz - clz) * inv_block - (0.75f + 1e-3f);
+        const int qhi = min((int)floorf(top), last_block), qlo = max((int)ceilf(bottom), 0);
+        if (qlo <= qhi) blocks = (2u << qhi) - (1u << qlo);
+      }
+      if (__ballot(blocks != 0) == 0) continue;
 #pragma unroll
       for (int q = 0; q < kBlocks; ++q) {
-        unsigned mq = (unsigned)(m >> (kPerRound * q)) & ((1u << kPerRound) - 1u);
-        // the record of a passing pair comes straight from the lane that tested it
+        unsigned long long mq = __ballot((blocks >> q) & 1u);
 #pragma unroll 1
         while (mq != 0) {                          // loses a bit per trip
-          const int src = q * kPerRound + __builtin_ctz(mq);
-          mq &= mq - 1u;
+          const int src = __builtin_ctzll(mq);
+          mq &= mq - 1ull;
           const float rx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.x), src));
           const float ry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.y), src));
           const float rz = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.z), src));
