@@ -367,6 +367,12 @@ splat_channel_kernel(
 
   if (sorted) {
     if (!column_live) return;
+    // Most or all workgroups of a launch are resident at once, and a wave's time grows with the
+    // atoms around its column: waves with many records get a higher issue priority, so that they
+    // finish less far behind the others.
+    if (ncand >= 384) __builtin_amdgcn_s_setprio(3);
+    else if (ncand >= 256) __builtin_amdgcn_s_setprio(2);
+    else if (ncand >= 128) __builtin_amdgcn_s_setprio(1);
     // Channels differ a lot in work (some hold most atoms, many hold none, and an empty channel is
     // stores only), so the waves start at different channels: at any time some compute while
     // others store.  The order of the channels does not matter to the sums.
