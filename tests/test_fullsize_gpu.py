@@ -93,3 +93,55 @@ def test_backward_full_batch(mg, workload):
     grads2 = torch.empty_like(grads)
     gm.backward_batch(off, c["centers"], moved, types, radii, diff * 2, grads2)
     assert torch.equal(grads2, grads * 2)
+
+
+def test_vector_types_full_size_properties(mg, monkeypatch):
+    """Configuration 3 at its full size (16 x 10,000 atoms into 28x96^3) without the oracle: the
+    grid is linear in the type vectors, one example of the batch equals its single launch, the
+    matrix-core kernel agrees with the column kernel, and a one-hot type vector gives the
+    index-typed grid."""
+    v = synth.vector_batch()
+    B = len(v["offsets"]) - 1
+    gm = mg.GridMaker(0.25, 23.75)
+    dims = gm.grid_dimensions(28)
+    coords, radii = dev(v["coords"]), dev(v["radii"])
+    w = dev(v["types"])
+    off = v["offsets"]
+
+    def grid(weights, rows=slice(0, B)):
+        n0, n1 = int(off[rows.start]), int(off[rows.stop])
+        o = torch.empty((rows.stop - rows.start,) + dims, device="cuda")
+        gm.forward_batch(off[rows.start:rows.stop + 1] - off[rows.start],
+                         v["centers"][rows], coords[n0:n1], weights[n0:n1], radii[n0:n1], o)
+        return o
+
+    full = grid(w)
+    assert float(full.min()) >= 0.0 and float(full.max()) > 0.5
+    # linear in the weights (scaling by a power of two is exact)
+    assert torch.equal(grid(0.5 * w, slice(3, 5)), 0.5 * full[3:5])
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    w2 = torch.rand(w.shape, device="cuda", generator=gen)
+    both = grid(w + w2, slice(6, 8))
+    parts = full[6:8] + grid(w2, slice(6, 8))
+    assert float((both - parts).abs().max()) <= 1e-6 + 2e-5 * float(parts.abs().max())
+    # an example of the batch is its single launch
+    s = slice(int(off[9]), int(off[10]))
+    one = torch.empty(dims, device="cuda")
+    gm.forward(tuple(v["centers"][9]), coords[s], w[s], radii[s], one)
+    assert torch.equal(one, full[9])
+    # the column kernel sums in atom order, the matrix cores four atoms at a time
+    monkeypatch.setenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", "1")
+    col = grid(w, slice(12, 14))
+    monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
+    err = (col - full[12:14]).abs()
+    assert float((err - 1e-5 * col.abs()).max()) <= 1e-6
+    # one-hot weights: the index-typed grid
+    types = torch.randint(0, 28, (int(off[1]),), device="cuda")
+    hot = torch.zeros((int(off[1]), 28), device="cuda")
+    hot[torch.arange(int(off[1]), device="cuda"), types] = 1.0
+    a = torch.empty(dims, device="cuda")
+    b = torch.empty(dims, device="cuda")
+    gm.forward(tuple(v["centers"][0]), coords[:int(off[1])], hot, radii[:int(off[1])], a)
+    gm.forward(tuple(v["centers"][0]), coords[:int(off[1])], types.float(), radii[:int(off[1])], b)
+    err = (a - b).abs()
+    assert float((err - 1e-5 * b.abs()).max()) <= 1e-6
