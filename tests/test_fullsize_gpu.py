@@ -145,3 +145,44 @@ def test_vector_types_full_size_properties(mg, monkeypatch):
     gm.forward(tuple(v["centers"][0]), coords[:int(off[1])], types.float(), radii[:int(off[1])], b)
     err = (a - b).abs()
     assert float((err - 1e-5 * b.abs()).max()) <= 1e-6
+
+
+def test_interpolation_full_size_properties(mg):
+    """Configuration 4 at its full size (50 x 28x48^3) without the oracle: the identity gives the
+    input back, a quarter turn about z through the grid centre is a permutation of the voxels,
+    resampling is linear in the input, and a batch equals its single launches."""
+    B, K, D = 50, 28, 48
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    src = torch.randn((B, K, D, D, D), device="cuda", generator=gen)
+    gi = mg.GridInterpolater(0.5, 23.5, 0.5, 23.5)
+    zeros = np.zeros((B, 3), np.float32)
+    ident = np.tile(np.asarray([1, 0, 0, 0], np.float32), (B, 1))
+    out = torch.empty_like(src)
+    gi.forward_batch(src, ident, zeros, zeros, out)
+    assert torch.equal(out, src)
+    # rotation by 90 degrees about z: (x, y, z) -> (-y, x, z); the grid is symmetric about its
+    # centre, so every output voxel is one input voxel (up to rounding of the rotated coordinate)
+    s = np.float32(np.sqrt(0.5))
+    turn = np.tile(np.asarray([s, 0, 0, s], np.float32), (B, 1))
+    gi.forward_batch(src, turn, zeros, zeros, out)
+    a = torch.rot90(src, 1, dims=(2, 3))
+    b = torch.rot90(src, -1, dims=(2, 3))
+    err = min(float((out - a).abs().max()), float((out - b).abs().max()))
+    assert err < 2e-4        # weights of 1 - O(1e-6) on values of a few units
+    # random transforms: linear in the input, and a batch is its single launches
+    rng = np.random.default_rng(40)
+    quats = synth.random_quaternions(rng, B)
+    trans = rng.uniform(-1.5, 1.5, (B, 3)).astype(np.float32)
+    gi.forward_batch(src, quats, zeros, trans, out)
+    other = torch.randn((4, K, D, D, D), device="cuda", generator=gen)
+    o1 = torch.empty_like(other)
+    o2 = torch.empty_like(other)
+    gi.forward_batch(other, quats[10:14], zeros[:4], trans[10:14], o1)
+    gi.forward_batch(0.5 * src[10:14] + other, quats[10:14], zeros[:4], trans[10:14], o2)
+    want = 0.5 * out[10:14] + o1
+    assert float((o2 - want).abs().max()) <= 1e-6 + 1e-5 * float(want.abs().max())
+    one = torch.empty((K, D, D, D), device="cuda")
+    for bidx in (0, 23, 49):
+        gi.forward(src[bidx], mg.Transform(mg.Quaternion(*[float(x) for x in quats[bidx]]),
+                                           (0, 0, 0), tuple(float(x) for x in trans[bidx])), one)
+        assert torch.equal(one, out[bidx])
