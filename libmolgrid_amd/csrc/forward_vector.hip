@@ -265,12 +265,11 @@ hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nb
                                  hipStream_t stream) {
   // per-atom radii take the column kernel; type-indexed radii and the exact-predicate modes
   // (truncated Gaussian) use the cubic-tile kernel below
-  // (densities: the matrix-core kernel; MOLGRID_HIP_VECTOR_COLUMN_KERNEL=1 keeps the column kernel,
-  // which binary occupancy always uses because its sums are compared bit for bit)
+  // (the matrix-core kernel; MOLGRID_HIP_VECTOR_COLUMN_KERNEL=1 keeps the column kernel)
   const char* column_only = getenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL");
-  if (!radii_type_indexed && !exact && !binary && !(column_only != nullptr && column_only[0] == '1'))
+  if (!radii_type_indexed && !exact && !(column_only != nullptr && column_only[0] == '1'))
     return launch_forward_vector_mfma(g, batch, nbatch, centers, coords, type_vector, radii, out,
-                                      stream);
+                                      binary, stream);
   if (!radii_type_indexed && !exact)
     return launch_forward_vector_column(g, batch, nbatch, centers, coords, type_vector, radii, out,
                                         binary, exact, stream);

@@ -16,9 +16,13 @@
 // as float4 pieces of whole z rows.  A wave keeps the 32 x 64 sums of each of its three blocks in
 // eight 4-register tiles: two halves of the channels by the four x planes of the 4x4x4 voxels.
 //
-// The matrix cores add the four products of a step to the running sum in their own order, so the
-// sums can differ from the CPU loop's in the last bits (well inside the density tolerance); binary
-// occupancy, which is compared bit for bit, stays on the column kernel.
+// Binary occupancy adds the weights themselves (density 1 where the atom covers the voxel, by the
+// reference's exact float comparison) and is compared bit for bit with the CPU loop, which adds
+// them in atom order.  v_mfma_f32_16x16x4f32 adds the four products of a step to the running sum
+// one after the other, each rounded to float32 -- measured: every binary comparison of the test
+// suite (sums of tens of weights in tens of thousands of voxels) is identical -- so the order of
+// the list, ascending atoms, is the order of the sum.  Densities differ from the column kernel in
+// the last bits only because dy^2 + dz^2 is shared by the four x planes here.
 #include <type_traits>
 
 #include "kernels.h"
@@ -50,6 +54,7 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+template <bool BINARY>
 __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void
 splat_vector_mfma_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
@@ -129,7 +134,7 @@ splat_vector_mfma_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int a = a0 + u * kWave + lane;
-        const float reach = rr[u] * g.radius_scale * g.frm;
+        const float reach = rr[u] * g.radius_scale * (BINARY ? 1.0f : g.frm);
         const bool p = (a < we) && box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy,
                                                  chz) <= reach * reach * kCullSlack;
         const unsigned long long m = __ballot(p);
@@ -167,7 +172,8 @@ splat_vector_mfma_kernel(
         ar = radii[a] * g.radius_scale;
         ar2 = ar * ar;
       }
-      s_rec[tid] = make_float4(coords[3 * a], coords[3 * a + 1], coords[3 * a + 2], 1.0f / ar2);
+      s_rec[tid] = make_float4(coords[3 * a], coords[3 * a + 1], coords[3 * a + 2],
+                               BINARY ? ar2 : 1.0f / ar2);
       s_recatom[tid] = a;
     }
     __syncthreads();
@@ -226,7 +232,7 @@ splat_vector_mfma_kernel(
               if (i < m) {
                 rec = s_rec[i];
                 const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
-                pass = d2 * rec.w <= frm2 * kCullSlack;
+                pass = BINARY ? (d2 <= rec.w * kCullSlack) : (d2 * rec.w <= frm2 * kCullSlack);
               }
               const unsigned long long bm = __ballot(pass);
               const int n = __popcll(bm);
@@ -264,7 +270,7 @@ splat_vector_mfma_kernel(
                 // a slot past the list has no reach at all, so its density is exactly zero (zero
                 // weight alone would not do: a stale record can give an infinite density, and
                 // 0 * inf is not a number)
-                const float rw = cur.have ? cur.r.w : INFINITY;
+                const float rw = cur.have ? cur.r.w : (BINARY ? -1.0f : INFINITY);
                 const float w0 = (cur.have && chan_live[0]) ? cur.w0 : 0.f;
                 const float w1 = (cur.have && chan_live[1]) ? cur.w1 : 0.f;
                 const float dy = vy - cur.r.y, dz = vz - cur.r.z;
@@ -272,12 +278,18 @@ splat_vector_mfma_kernel(
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                   const float dx = vx[t] - cur.r.x;
-                  const float u = (dx * dx + dyz2) * rw;
-                  const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
-                  const float su = __builtin_amdgcn_sqrtf(u);
-                  const float quadr = fmaxf(fmaf(g.A, u, fmaf(g.B, su, g.C)), 0.f);
-                  float d = (u <= grm2) ? gauss : quadr;
-                  d = (u <= frm2) ? d : 0.f;
+                  float d;
+                  if (BINARY) {
+                    // the reference's own float sequence ((dx^2 + dy^2) + dz^2) < ar^2
+                    d = sq_distance_exact(dx, dy, dz) < rw ? 1.0f : 0.0f;
+                  } else {
+                    const float u = (dx * dx + dyz2) * rw;
+                    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                    const float su = __builtin_amdgcn_sqrtf(u);
+                    const float quadr = fmaxf(fmaf(g.A, u, fmaf(g.B, su, g.C)), 0.f);
+                    d = (u <= grm2) ? gauss : quadr;
+                    d = (u <= frm2) ? d : 0.f;
+                  }
                   sums[blk][t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w0, d, sums[blk][t][0], 0, 0, 0);
                   sums[blk][t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w1, d, sums[blk][t][1], 0, 0, 0);
                 }
@@ -364,16 +376,21 @@ splat_vector_mfma_kernel(
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
                                       const Vec3Arg& centers, const float* coords,
                                       const float* type_vector, const float* radii, float* out,
-                                      hipStream_t stream) {
+                                      bool binary, hipStream_t stream) {
   const int cols_per_side = (g.dim + kColXY - 1) / kColXY;
   const int slabs = (g.dim + kSlabZ - 1) / kSlabZ;
   const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
   const int vec_store = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0) &&
                          ((chan_stride * g.ntypes) % 4 == 0)) ? 1 : 0;
   const int groups = cols_per_side * ((cols_per_side + kColsPerGroup - 1) / kColsPerGroup);
-  hipLaunchKernelGGL(splat_vector_mfma_kernel, dim3(groups * slabs, nbatch), dim3(kColThreads), 0,
-                     stream, g, batch, centers, coords, type_vector, radii, out, cols_per_side,
-                     vec_store);
+  if (binary)
+    hipLaunchKernelGGL(splat_vector_mfma_kernel<true>, dim3(groups * slabs, nbatch),
+                       dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
+                       out, cols_per_side, vec_store);
+  else
+    hipLaunchKernelGGL(splat_vector_mfma_kernel<false>, dim3(groups * slabs, nbatch),
+                       dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
+                       out, cols_per_side, vec_store);
   return hipGetLastError();
 }
 

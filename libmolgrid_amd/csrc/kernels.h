@@ -47,7 +47,7 @@ hipError_t launch_forward_vector_column(const GridArg& g, const BatchArg& batch,
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
                                       const Vec3Arg& centers, const float* coords,
                                       const float* type_vector, const float* radii, float* out,
-                                      hipStream_t stream);
+                                      bool binary, hipStream_t stream);
 
 hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
                                  const Vec3Arg& centers, const float* coords,

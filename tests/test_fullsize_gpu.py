@@ -135,6 +135,18 @@ def test_vector_types_full_size_properties(mg, monkeypatch):
     monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
     err = (col - full[12:14]).abs()
     assert float((err - 1e-5 * col.abs()).max()) <= 1e-6
+    # binary occupancy (sums of weights, about 35 per voxel): the two kernels agree bit for bit
+    gmb = mg.GridMaker(0.25, 23.75, True)
+    n0, n1 = int(off[12]), int(off[14])
+    bin_mfma = torch.empty((2,) + dims, device="cuda")
+    gmb.forward_batch(off[12:15] - off[12], v["centers"][12:14], coords[n0:n1], w[n0:n1],
+                      radii[n0:n1], bin_mfma)
+    monkeypatch.setenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", "1")
+    bin_col = torch.empty((2,) + dims, device="cuda")
+    gmb.forward_batch(off[12:15] - off[12], v["centers"][12:14], coords[n0:n1], w[n0:n1],
+                      radii[n0:n1], bin_col)
+    monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
+    assert torch.equal(bin_mfma, bin_col) and float(bin_col.max()) > 1.0
     # one-hot weights: the index-typed grid
     types = torch.randint(0, 28, (int(off[1]),), device="cuda")
     hot = torch.zeros((int(off[1]), 28), device="cuda")
