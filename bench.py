@@ -39,6 +39,25 @@ def event_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def step_breakdown(fns, iters):
+    """Average milliseconds of each launch of a step when the launches follow each other as in the
+    timed loop (events between them on the launch stream).  A kernel timed alone over and over
+    finds part of its input in the last-level cache from its previous run; inside the step the
+    forward pass has just written 619 MB through that cache."""
+    import torch
+    rows = [[torch.cuda.Event(enable_timing=True) for _ in range(len(fns) + 1)]
+            for _ in range(iters)]
+    torch.cuda.synchronize()
+    for row in rows:
+        row[0].record()
+        for fn, ev in zip(fns, row[1:]):
+            fn()
+            ev.record()
+    torch.cuda.synchronize()
+    return [sum(row[i].elapsed_time(row[i + 1]) for row in rows) / iters
+            for i in range(len(fns))]
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary
     (FETCH_SIZE + WRITE_SIZE, KiB per dispatch; calibration factor 1.0, stated in that file).
@@ -238,6 +257,7 @@ def main():
     ms_fwd = event_ms(k_forward, it)
     ms_bwd = event_ms(k_backward, it)
     ms_tr = event_ms(k_transform, it)
+    in_step = step_breakdown([k_transform, k_forward, k_backward, k_unrotate], it)
 
     grid_bytes = B * T * D ** 3 * 4
     fwd_bytes = grid_bytes + n_atoms * 20          # grid written once + coords/type/radius read
@@ -259,12 +279,13 @@ def main():
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
     }
     kernels = {
-        "forward": {"ms": round(ms_fwd, 4), "grids_per_s": round(B / (ms_fwd * 1e-3), 1),
+        "forward": {"ms": round(ms_fwd, 4), "in_step_ms": round(in_step[1], 4), "grids_per_s": round(B / (ms_fwd * 1e-3), 1),
                     "GBps": round(fwd_gbs, 1), "hbm_frac": round(fwd_gbs / HBM_PEAK_GBS, 4)},
-        "backward": {"ms": round(ms_bwd, 4),
+        "backward": {"ms": round(ms_bwd, 4), "in_step_ms": round(in_step[2], 4),
                      "atom_grads_per_s": round(n_atoms / (ms_bwd * 1e-3), 1),
                      "GBps": round(bwd_gbs, 1), "hbm_frac": round(bwd_gbs / HBM_PEAK_GBS, 4)},
-        "transform": {"ms": round(ms_tr, 4)},
+        "transform": {"ms": round(ms_tr, 4), "in_step_ms": round(in_step[0], 4),
+                      "unrotate_in_step_ms": round(in_step[3], 4)},
     }
 
     if not args.no_extras:
