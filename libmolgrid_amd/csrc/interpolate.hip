@@ -71,7 +71,6 @@ constexpr int kVox = kTileX * kTileY * kTileZ / kTileThreads;
 constexpr int kWin = 21;                       // largest staged window side
 constexpr int kWinZ = 22;                      // z stride of the window in LDS (even: 8-byte pairs)
 constexpr int kWinSize = kWin * kWin * kWinZ;  // floats per buffer
-constexpr int kStagePer = (kWin * kWin * kWin + kTileThreads - 1) / kTileThreads;  // 19
 constexpr int kFewRounds = 6;                  // staged elements per thread and channel (6 x 512 >= 2,800)
 // longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
 constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
@@ -82,7 +81,7 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     Vec3Arg out_centers, float* __restrict__ out, int plain_staging) {
   extern __shared__ __align__(16) float s_win[];   // two buffers of kWinSize floats, one spare slot
   __shared__ float s_lo[3], s_hi[3];
-  __shared__ int s_scan[kStagePer * kTileWaves + 1];
+  __shared__ int s_scan[kTileWaves];
 
   // workgroup -> (example, tile): consecutive workgroups are dealt round-robin to the 8 XCDs, so
   // example b is pinned to XCD b % 8 and its tiles run there in z-fastest order
@@ -182,104 +181,74 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     __syncthreads();
   }
 
-  // ---- staging plan of this thread: up to kStagePer window elements per channel ---------------
+  // ---- staging plan: the window positions in use, in window order, dealt out evenly ------------
   // Window positions outside the input grid hold zero for every channel: both buffers are cleared
-  // once and such positions, the positions no tap reads and the unused tail of the plan are
-  // steered to a spare LDS slot and to element 0 of the channel, so that the per-channel loop is
-  // load + write without tests.
+  // once and such positions, the positions no tap reads and the unused tail of a thread's share
+  // are steered to a spare LDS slot and to element 0 of the channel, so that the per-channel loop
+  // is load + write without tests.
+  // One thread per (x, y) row of the window (at most 21 x 21 of them) collects, as a bit mask,
+  // the z positions of its row that some tap reads and the input grid holds; a prefix sum over the
+  // workgroup numbers them in window order, so neighbouring slots are neighbouring addresses; the
+  // (source offset, LDS cell) pairs go to a list in the window's LDS and are read back strided by
+  // the workgroup size: every thread gets an equal share.
   const int wcount = wn[0] * wn[1] * wn[2];
   const int plane = wn[1] * wn[2];
-  const int rounds = (wcount + kTileThreads - 1) / kTileThreads;   // uniform: rounds in use
-  const float inv_plane = 1.0f / (float)plane, inv_row = 1.0f / (float)wn[2];
-  int st_src[kStagePer];   // offset inside one input channel
-  int st_dst[kStagePer];   // offset inside the LDS window
-#pragma unroll
-  for (int e = 0; e < kStagePer; ++e) {
-    const int n = tid + e * kTileThreads;
-    st_dst[e] = 2 * kWinSize;   // the spare slot
-    st_src[e] = 0;
-    if (e < rounds && n < wcount) {
-      // n = (ex * wn[1] + ey) * wn[2] + ez; quotients by float reciprocal, corrected by one step
-      int ex = (int)((float)n * inv_plane);
-      ex -= (ex * plane > n) ? 1 : 0;
-      ex += ((ex + 1) * plane <= n) ? 1 : 0;
-      const int r = n - ex * plane;
-      int ey = (int)((float)r * inv_row);
-      ey -= (ey * wn[2] > r) ? 1 : 0;
-      ey += ((ey + 1) * wn[2] <= r) ? 1 : 0;
-      const int ez = r - ey * wn[2];
-      const int gx = wlo[0] + ex, gy = wlo[1] + ey, gz = wlo[2] + ez;
-      const int cell = (ex * kWin + ey) * kWinZ + ez;
-      if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id &&
-          reinterpret_cast<const unsigned char*>(s_win)[cell] != 0) {
-        st_dst[e] = cell;
-        st_src[e] = (gx * id + gy) * id + gz;
+  const int lane = tid & 63, wave = tid >> 6;
+  unsigned zmask = 0;
+  int row_cell = 0, row_src = 0;
+  if (tid < wn[0] * wn[1]) {
+    const int ex = tid / wn[1], ey = tid - ex * wn[1];
+    const int gx = wlo[0] + ex, gy = wlo[1] + ey;
+    row_cell = (ex * kWin + ey) * kWinZ;
+    row_src = (gx * id + gy) * id + wlo[2];
+    if (gx >= 0 && gx < id && gy >= 0 && gy < id) {
+      const unsigned char* used = reinterpret_cast<const unsigned char*>(s_win) + row_cell;
+      for (int ez = 0; ez < wn[2]; ++ez) {
+        const int gz = wlo[2] + ez;
+        if (gz >= 0 && gz < id && used[ez] != 0) zmask |= 1u << ez;
       }
     }
   }
-  // ---- the planned elements, compacted: every thread gets an equal share of the ones in use --
-  // Slots are numbered in window order (round, wave, lane), so neighbouring lanes still load
-  // neighbouring addresses.  Counts per (round, wave) go to LDS, wave 0 turns them into offsets,
-  // the (source, destination) pairs are written to a list in the window's LDS and read back
-  // strided by the workgroup size.
-  int* counts = reinterpret_cast<int*>(s_scan);            // [kStagePer][kTileWaves] + total
-  const int lane = tid & 63, wave = tid >> 6;
-  int before[kStagePer];                                   // planned elements of the wave before this lane
+  const int mine = __popc(zmask);
+  int incl = mine;                                         // inclusive scan over the wave
 #pragma unroll
-  for (int e = 0; e < kStagePer; ++e) {
-    const unsigned long long m = __ballot(st_dst[e] != 2 * kWinSize);
-    before[e] = __popcll(m & ((1ull << lane) - 1ull));
-    if (lane == 0) counts[e * kTileWaves + wave] = __popcll(m);
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
   }
-  __syncthreads();   // counts complete; every thread has read the marks
-  if (wave == 0) {
-    constexpr int kCounts = kStagePer * kTileWaves;        // 152
-    constexpr int kPerLane = (kCounts + 63) / 64;          // 3
-    int mine[kPerLane], sum = 0;
+  if (lane == 63) s_scan[wave] = incl;
+  __syncthreads();   // wave totals complete; every thread has read the marks
+  int slot0 = incl - mine, planned = 0;
 #pragma unroll
-    for (int q = 0; q < kPerLane; ++q) {
-      const int i = lane * kPerLane + q;
-      mine[q] = i < kCounts ? counts[i] : 0;
-      sum += mine[q];
-    }
-    int incl = sum;                                        // inclusive scan over the lanes
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(incl, d);
-      if (lane >= d) incl += up;
-    }
-    int run = incl - sum;
-#pragma unroll
-    for (int q = 0; q < kPerLane; ++q) {
-      const int i = lane * kPerLane + q;
-      if (i < kCounts) counts[i] = run;
-      run += mine[q];
-    }
-    if (lane == 63) counts[kCounts] = incl;
+  for (int w = 0; w < kTileWaves; ++w) {
+    const int c = s_scan[w];
+    slot0 += w < wave ? c : 0;
+    planned += c;
   }
-  __syncthreads();
   {
     int* list = reinterpret_cast<int*>(s_win);             // pairs: source offset, destination
-#pragma unroll
-    for (int e = 0; e < kStagePer; ++e) {
-      if (st_dst[e] != 2 * kWinSize) {
-        const int slot = counts[e * kTileWaves + wave] + before[e];
-        list[2 * slot] = st_src[e];
-        list[2 * slot + 1] = st_dst[e];
-      }
+    unsigned m = zmask;
+    int slot = slot0;
+    while (m != 0) {
+      const int ez = __builtin_ctz(m);
+      m &= m - 1u;
+      list[2 * slot] = row_src + ez;
+      list[2 * slot + 1] = row_cell + ez;
+      ++slot;
     }
   }
   __syncthreads();
-  const int planned = counts[kStagePer * kTileWaves];
   const int rounds_used = (planned + kTileThreads - 1) / kTileThreads;   // uniform
+  int st_src[kFewRounds];   // offset inside one input channel
+  int st_dst[kFewRounds];   // offset inside the LDS window
   {
     const int* list = reinterpret_cast<const int*>(s_win);
 #pragma unroll
     for (int e = 0; e < kFewRounds; ++e) {
       const int slot = tid + e * kTileThreads;
-      const bool mine = slot < planned;
-      st_src[e] = mine ? list[2 * slot] : 0;
-      st_dst[e] = mine ? list[2 * slot + 1] : 2 * kWinSize;
+      const bool have = slot < planned;
+      st_src[e] = have ? list[2 * slot] : 0;
+      st_dst[e] = have ? list[2 * slot + 1] : 2 * kWinSize;
     }
   }
   __syncthreads();   // every thread holds its share: the window can be cleared
