@@ -277,6 +277,10 @@ def main():
                                     else "backward_index_kernel"),
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
+        # the same kernel between the other launches of the step (see step_breakdown)
+        "in_step_ms": round(in_step[1] if dominant_fwd else in_step[2], 4),
+        "in_step_frac": round((fwd_bytes / in_step[1] if dominant_fwd else bwd_bytes / in_step[2])
+                              / 1e6 / HBM_PEAK_GBS, 4),
     }
     kernels = {
         "forward": {"ms": round(ms_fwd, 4), "in_step_ms": round(in_step[1], 4), "grids_per_s": round(B / (ms_fwd * 1e-3), 1),
