@@ -292,22 +292,50 @@ splat_channel_kernel(
         const int qhi = min((int)floorf(top), last_block), qlo = max((int)ceilf(bottom), 0);
         if (qlo <= qhi) blocks = (2u << qhi) - (1u << qlo);
       }
-      if (__ballot(blocks != 0) == 0) continue;
-#pragma unroll
-      for (int q = 0; q < kBlocks; ++q) {
-        unsigned long long mq = __ballot((blocks >> q) & 1u);
+      // the records that reach the column, in record order; the part of the distance that lies in
+      // x and y is the same for every block of a record
+      unsigned long long todo = __ballot(blocks != 0);
 #pragma unroll 1
-        while (mq != 0) {                          // loses a bit per trip
-          const int src = __builtin_ctzll(mq);
-          mq &= mq - 1ull;
-          const float rx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.x), src));
-          const float ry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.y), src));
-          const float rz = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.z), src));
-          const float rw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.w), src));
-          float val;
-          const bool hit = density_hit<BINARY, false>(g, vx - rx, vy - ry, vz[q] - rz, rw, 0.f, frm2,
-                                                      grm2, quad_c, val);
-          if (hit) acc[q] = BINARY ? 1.0f : acc[q] + val;
+      while (todo != 0) {                          // loses a bit per trip
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1ull;
+        const float rx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.x), src));
+        const float ry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.y), src));
+        const float rz = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.z), src));
+        const float rw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(rec.w), src));
+        const unsigned reach = (unsigned)__builtin_amdgcn_readlane((int)blocks, src);
+        const float dx = vx - rx, dy = vy - ry;
+        float dxy2;
+        if (BINARY) {
+#pragma clang fp contract(off)
+          dxy2 = dx * dx + dy * dy;
+        } else {
+          dxy2 = fmaf(dx, dx, dy * dy);
+        }
+#pragma unroll
+        for (int q0 = 0; q0 < kBlocks; q0 += 4) {
+          if (((reach >> q0) & 0xfu) == 0) continue;
+#pragma unroll
+          for (int q = q0; q < q0 + 4; ++q) {
+            if (((reach >> q) & 1u) == 0) continue;
+            const float dz = vz[q] - rz;
+            if (BINARY) {
+              float rsq;
+              {
+#pragma clang fp contract(off)
+                rsq = dxy2 + dz * dz;
+              }
+              if (rsq < rw) acc[q] = 1.0f;
+            } else {
+              const float u = fmaf(dz, dz, dxy2) * rw;
+              if (u <= frm2) {
+                const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                const float su = __builtin_amdgcn_sqrtf(u);
+                const float quad = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+                acc[q] += (u <= grm2) ? gauss : quad;
+              }
+            }
+          }
         }
       }
     }
