@@ -41,9 +41,9 @@ def event_ms(fn, iters):
 
 def step_breakdown(fns, iters):
     """Average milliseconds of each launch of a step when the launches follow each other as in the
-    timed loop (events between them on the launch stream).  A kernel timed alone over and over
-    finds part of its input in the last-level cache from its previous run; inside the step the
-    forward pass has just written 619 MB through that cache."""
+    timed loop (events between them on the launch stream).  A check on the per-kernel figures: a
+    kernel that leaves dirty lines in the last-level cache looks shorter here than launched alone
+    and the kernel after it longer."""
     import torch
     rows = [[torch.cuda.Event(enable_timing=True) for _ in range(len(fns) + 1)]
             for _ in range(iters)]

@@ -167,7 +167,9 @@ splat_channel_kernel(
         if (from_stage) v = *reinterpret_cast<const v4f*>(stage + st_lds + k * 4 * kRowPad);
         const unsigned off = chan_off + st_off + k * st_xstride;
         if (aligned_rows && st_gz + 3 < dim) {
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf, (int)off, 0, 0);
+          // non-temporal: nothing reads the grids back soon enough to find them in the last-level
+          // cache, and without the hint its write-back runs on into the next kernel
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf, (int)off, 0, 2);
         } else {
           const float e[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
