@@ -324,7 +324,9 @@ splat_vector_mfma_kernel(
             float* dst = ob + (size_t)st_chan[k] * chan_stride + st_sp[k];
             const int gz = z0 + ((tid + k * kColThreads) % 12) * 4;
             if ((vec_store & 1) && gz + 3 < dim) {
-              *reinterpret_cast<v4f*>(dst) = v;
+              // non-temporal: the grids are not read back soon, and the write-back of plain
+              // stores runs on into the next launch (binary occupancy: 0.65 ms against 0.85 ms)
+              __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(dst));
             } else {
               dst[0] = v.x;
               if (gz + 1 < dim) dst[1] = v.y;
