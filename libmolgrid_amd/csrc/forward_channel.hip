@@ -270,9 +270,9 @@ splat_channel_kernel(
   // ---- records [lo, hi) of s_rec, all of one channel, added to the sums -----------------------
   // A cull round takes 64 records, one per lane: the lane finds the interval of z the atom can
   // reach inside the column (its reach shrunk by the distance to the column's footprint in x and
-  // y) and from it the range of blocks, as a bit mask.  One ballot per block then gives the
-  // records of that block, which are taken in record order; the atom's record comes straight from
-  // the lane that tested it.
+  // y) and from it the range of blocks, as a bit mask.  The records that reach the column are then
+  // taken one at a time, in record order, each over the blocks of its mask; the record comes
+  // straight from the lane that tested it.
   const float inv_block = 0.25f / g.resolution;             // blocks per unit length along z
   const int last_block = (zend - z0 + 3) / 4 - 1;
   auto splat_records = [&](int lo, int hi) {
