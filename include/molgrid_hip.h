@@ -11,10 +11,13 @@
  *   - Every array pointer is a DEVICE pointer on the current HIP device unless
  *     its name ends in `_host`.  Arrays are dense, row-major, float32.
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Work
- *     is enqueued asynchronously; no entry point synchronises or allocates.
+ *     is enqueued asynchronously; no entry point synchronises, and none allocates
+ *     except mg_forward_index (see there).
  *   - Batches: example b owns atoms [atom_offsets[b], atom_offsets[b+1]) of the
- *     packed atom arrays.  When `atom_offsets` is NULL every example owns
- *     `atoms_per_example` consecutive atoms (the reference's padded BxN layout,
+ *     packed atom arrays, and `atoms_per_example` must then be at least the size
+ *     of the largest example (it sizes launches and workspaces).  When
+ *     `atom_offsets` is NULL every example owns `atoms_per_example` consecutive
+ *     atoms (the reference's padded BxN layout,
  *     include/libmolgrid/grid_maker.h:265-301; nbatch = 1 is the un-batched
  *     call).  Per-example float3/float4 parameters (`centers`, `quats`, ...)
  *     are device arrays with one row per example; when such a pointer is NULL
@@ -94,11 +97,33 @@ int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per
                           int dotranslate, const float* in_coords, float* out_coords,
                           void* stream);
 
-/* GridMaker::forward, index types; replaces forward_gpu and its launcher
- * (src/grid_maker.cu:212-289) for a whole batch in one launch, with the values
- * of the CPU overload (src/grid_maker.cpp:153-212).
+/* GridMaker::forward, index types; replaces the cudaMemset + forward_gpu launch
+ * per example (src/grid_maker.cu:212-289) for a whole batch, with the values of
+ * the CPU overload (src/grid_maker.cpp:153-212).
  *   coords [n,3], type_index [n], radii [n], out [nbatch, ntypes, dim, dim, dim]
- * `out` is overwritten completely (no memset needed before the call). */
+ * `out` is overwritten completely (no memset needed before the call).  Two
+ * launches: the atoms are sorted by channel into `workspace` (device memory,
+ * at least mg_forward_index_workspace_size() bytes, 256-byte aligned, contents
+ * undefined before and after), then splatted.  Calls that run concurrently need
+ * a workspace each.  MG_ERR_UNSUPPORTED: a channel of 4 GB or more, or
+ * nbatch * atoms_per_example >= 2^28. */
+int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                        int atoms_per_example, const float* grid_centers,
+                        const float grid_center_host[3], const float* coords,
+                        const float* type_index, const float* radii, int ntypes, float* out,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Host only.  Bytes of workspace mg_forward_index_ws needs for these sizes (0
+ * for an empty call). */
+size_t mg_forward_index_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
+                                       int ntypes);
+
+/* The same with a workspace that the library keeps per device: it is allocated
+ * (hipMalloc) by the first call on a device and replaced (hipFree + hipMalloc,
+ * which wait for the device) when a call needs a larger one; it is never
+ * released.  All calls on one device share it, so calls on different streams of
+ * one device must not overlap.  Callers that must not allocate, or that use
+ * several streams, take mg_forward_index_ws. */
 int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                      int atoms_per_example, const float* grid_centers,
                      const float grid_center_host[3], const float* coords,

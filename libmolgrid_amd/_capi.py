@@ -17,7 +17,8 @@ MG_ERR_NULL_POINTER = -4
 
 EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
-    "mg_transform_backward", "mg_forward_index", "mg_forward_vector", "mg_backward_index",
+    "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
+    "mg_forward_index_workspace_size", "mg_forward_vector", "mg_backward_index",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate",
 )
 
@@ -63,6 +64,9 @@ def _load():
     lib.mg_transform_backward.argtypes = tr
     fwd = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp]
     lib.mg_forward_index.argtypes = fwd
+    lib.mg_forward_index_ws.argtypes = fwd[:-1] + [_vp, ctypes.c_size_t, _vp]
+    lib.mg_forward_index_workspace_size.argtypes = [gm, _i, _i, _i]
+    lib.mg_forward_index_workspace_size.restype = ctypes.c_size_t
     lib.mg_forward_vector.argtypes = fwd
     lib.mg_backward_index.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp, _vp]
     lib.mg_backward_vector.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,
@@ -75,7 +79,7 @@ def _load():
                                    _vp, _f3, _vp, _f3, _vp, _vp]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)
-        if name not in ("mg_error_string",):
+        if name not in ("mg_error_string", "mg_forward_index_workspace_size"):
             fn.restype = _i
     return lib
 

@@ -1,7 +1,9 @@
-// C ABI of the gridding library: argument checks, then one kernel launch per
-// call on the caller's stream.  Nothing here allocates or synchronises.
+// C ABI of the gridding library: argument checks, then the kernel launches of the call on the
+// caller's stream.  Nothing here synchronises; the only allocation is the workspace that
+// mg_forward_index keeps per device (mg_forward_index_ws takes the caller's instead).
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 #include "kernels.h"
 #include "molgrid_hip.h"
@@ -72,7 +74,7 @@ int from_hip(hipError_t e) { return e == hipSuccess ? MG_OK : (int)e; }
 
 extern "C" {
 
-int mg_version(void) { return 100; }
+int mg_version(void) { return 200; }
 
 const char* mg_error_string(int code) {
   switch (code) {
@@ -150,25 +152,110 @@ int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per
                                    in_coords, out_coords, (hipStream_t)stream));
 }
 
+namespace {
+
+int check_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                        int atoms_per_example, const float* coords, const float* type_index,
+                        const float* radii, int ntypes, const float* out, bool* nothing_to_do) {
+  *nothing_to_do = false;
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  // src/grid_maker.cpp:160-162
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (atoms_per_example < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || ntypes == 0) {
+    *nothing_to_do = true;
+    return MG_OK;
+  }
+  if (out == nullptr) return MG_ERR_NULL_POINTER;
+  const bool has_atoms = atoms_per_example > 0;
+  if (has_atoms && (coords == nullptr || type_index == nullptr || radii == nullptr))
+    return MG_ERR_NULL_POINTER;
+  return MG_OK;
+}
+
+int forward_index_with(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                       int atoms_per_example, const float* grid_centers,
+                       const float grid_center_host[3], const float* coords,
+                       const float* type_index, const float* radii, int ntypes, float* out,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  BatchArg batch{atom_offsets, atoms_per_example};
+  const hipError_t e = launch_forward_sorted(
+      grid_arg(g, ntypes), batch, nbatch, vec3(grid_centers, grid_center_host), coords, type_index,
+      radii, out, g->binary != 0, needs_exact(g), workspace, workspace_bytes, (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return MG_ERR_UNSUPPORTED;
+  return from_hip(e);
+}
+
+// Workspace of mg_forward_index, one per device, grown when a call needs more.
+struct DeviceWorkspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+constexpr int kMaxDevices = 64;
+DeviceWorkspace g_workspace[kMaxDevices];
+std::mutex g_workspace_mutex;
+
+}  // namespace
+
+size_t mg_forward_index_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
+                                       int ntypes) {
+  if (g == nullptr || nbatch <= 0 || ntypes <= 0 || atoms_per_example < 0) return 0;
+  return forward_sorted_workspace_bytes(nbatch, atoms_per_example, ntypes, (int)g->dim);
+}
+
+int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                        int atoms_per_example, const float* grid_centers,
+                        const float grid_center_host[3], const float* coords,
+                        const float* type_index, const float* radii, int ntypes, float* out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  bool nothing = false;
+  const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
+                                    radii, ntypes, out, &nothing);
+  if (s != MG_OK || nothing) return s;
+  if (workspace == nullptr) return MG_ERR_NULL_POINTER;
+  if (workspace_bytes < mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes))
+    return MG_ERR_INVALID_ARGUMENT;
+  return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
+                            grid_center_host, coords, type_index, radii, ntypes, out, workspace,
+                            workspace_bytes, stream);
+}
+
 int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                      int atoms_per_example, const float* grid_centers,
                      const float grid_center_host[3], const float* coords,
                      const float* type_index, const float* radii, int ntypes, float* out,
                      void* stream) {
-  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
-  if (s != MG_OK) return s;
-  // src/grid_maker.cpp:160-162
-  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || ntypes == 0) return MG_OK;
-  if (out == nullptr) return MG_ERR_NULL_POINTER;
-  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
-  if (has_atoms && (coords == nullptr || type_index == nullptr || radii == nullptr))
-    return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
-  return from_hip(launch_forward_index(grid_arg(g, ntypes), batch, nbatch,
-                                       vec3(grid_centers, grid_center_host), coords, type_index,
-                                       radii, out, g->binary != 0, needs_exact(g),
-                                       (hipStream_t)stream));
+  bool nothing = false;
+  const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
+                                    radii, ntypes, out, &nothing);
+  if (s != MG_OK || nothing) return s;
+  const size_t need = mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes);
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return from_hip(e);
+  if (dev < 0 || dev >= kMaxDevices) return MG_ERR_UNSUPPORTED;
+  void* workspace = nullptr;
+  size_t bytes = 0;
+  {
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    DeviceWorkspace& w = g_workspace[dev];
+    if (w.bytes < need) {
+      // hipFree waits for the device, so no launch is still using the old block
+      if (w.ptr != nullptr) (void)hipFree(w.ptr);
+      w.ptr = nullptr;
+      w.bytes = 0;
+      const size_t want = need + need / 2;
+      e = hipMalloc(&w.ptr, want);
+      if (e != hipSuccess) return from_hip(e);
+      w.bytes = want;
+    }
+    workspace = w.ptr;
+    bytes = w.bytes;
+  }
+  return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
+                            grid_center_host, coords, type_index, radii, ntypes, out, workspace, bytes,
+                            stream);
 }
 
 int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,

@@ -1,0 +1,690 @@
+// Forward splat for index types (GridMaker::forward, src/grid_maker.cpp:153-212,
+// src/grid_maker.cu:95-130), in two launches.
+//
+// 1. sort_atoms_kernel: the atoms of every example become 16-byte records (x, y, z, ar =
+//    radius * radius_scale), sorted by (channel, x slab of the centre) and, within a key, in
+//    ascending atom order (a stable counting sort, one workgroup per example).  Atoms without a
+//    channel drop out.  The workgroup also finds the rank of its example by size and writes the
+//    example's tables -- grid origin, example number, and for every (channel, x slab) the run of
+//    records that can reach the slab -- at that rank, so that the second launch meets the examples
+//    largest first.
+// 2. splat_sorted_kernel: one wave per work item, no workgroup of more than one wave, nothing
+//    shared between waves.  An item is a territory of 4 x (4 * COLS) x 48 voxels -- COLS columns
+//    of 4 x 4 voxels in (x, y), consecutive in y, each twelve 4x4x4 blocks tall -- of one example,
+//    for every R-th channel.  For each of these channels the first launch has left the run of
+//    records whose atoms can reach the territory's four x planes.  The wave first writes zeros for
+//    its channels with an empty run.  Then it walks the others: the records are read 64 at a time
+//    (one per lane, the next 64 in flight), each lane finds the blocks its record can reach, the
+//    records that reach the territory are taken one at a time, in record order, and summed in
+//    registers (one voxel of every block per lane); each column then goes through the wave's LDS
+//    stage and is written out as whole z rows.  The hardware hands out the items in order, the
+//    largest example first, so the last ones running are small.
+//
+// Sums run in record order: by x slab of the atom's centre, then by atom number.  That is a fixed
+// order (results are the same from run to run) but not the CPU loop's plain atom order, so
+// Gaussian densities agree with it to rounding, not to the bit; binary densities are exact.
+//
+// Every global access of the splat kernel goes through buffer instructions that carry the
+// extent of the array they address: an index outside it reads zero or is dropped.
+#include <algorithm>
+#include <cstdlib>
+
+#include "kernels.h"
+#include "splat_common.h"
+
+namespace mg {
+namespace {
+
+constexpr int kColXY = 4;                        // column footprint in x and y
+constexpr int kBlocks = 12;                      // 4x4x4 blocks of a column
+constexpr int kSlabZ = kBlocks * 4;              // 48
+constexpr int kRowPad = 52;                      // staged z row, padded against bank conflicts
+constexpr int kPlane = 16 * kRowPad;             // one staged column (floats)
+constexpr int kPieces = 16 * (kSlabZ / 4) / kWave;   // float4 pieces of a column per lane: 3
+constexpr int kBufferFlags = 0x00020000;         // untyped 32-bit elements, no swizzle
+constexpr int kItemChannels = 4;                 // channels an item takes, about
+constexpr int kItemChannelsMax = 64;             // ... and at most (one per lane)
+
+constexpr int kSortWaves = 16;
+constexpr int kSortThreads = kSortWaves * kWave;
+constexpr int kKeyGroup = 512;                   // keys a workgroup of the sort handles, at most
+constexpr int kCached = 4;                       // atoms a thread keeps in registers
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float uniform(float v) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void* p, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           (int)(bytes < 0xffffffffull ? bytes : 0xffffffffull),
+                                           kBufferFlags);
+}
+__device__ __forceinline__ float lane_value(float v, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+
+// ------------------------------------------------------------------------------------------
+// Workspace: slot_info [nbatch] | cand [nbatch * ntypes * nxs * 2] | records [capacity]
+// A key is (channel, x slab), where the slab of an atom is the group of four x planes its centre
+// lies in (clamped to the grid); nxs slabs.
+// ------------------------------------------------------------------------------------------
+constexpr size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct SortedAtoms {
+  float4* slot_info;   // per launch slot (examples in descending size): grid origin, example number
+  int* cand;           // per launch slot, channel and x slab: first and one-past-last record of the
+                       // channel that can reach the slab's four x planes
+  float4* records;
+  int capacity;        // records
+};
+
+SortedAtoms carve(void* workspace, int nbatch, int nkeys, long long capacity) {
+  unsigned char* p = static_cast<unsigned char*>(workspace);
+  SortedAtoms s;
+  s.slot_info = reinterpret_cast<float4*>(p);
+  p += align256((size_t)nbatch * 16);
+  s.cand = reinterpret_cast<int*>(p);
+  p += align256((size_t)nbatch * nkeys * 8);
+  s.records = reinterpret_cast<float4*>(p);
+  s.capacity = (int)capacity;
+  return s;
+}
+
+// slab of an x coordinate, as a float in [0, nxs - 1]; monotone in x
+__device__ __forceinline__ float slab_of(float x, float ox, float inv_slab, int nxs) {
+  return fminf(fmaxf(floorf((x - ox) * inv_slab + 0.125f), 0.f), (float)(nxs - 1));
+}
+
+// ------------------------------------------------------------------------------------------
+// Launch 1: a stable counting sort of the atoms by key.  Workgroup (part, example) takes the
+// channels [part * per_part, (part + 1) * per_part) of its example: it reads all atoms of the
+// example, counts those of lower channels (their records come first), and sorts its own.
+// per_part * nxs <= kKeyGroup.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
+    GridArg g, BatchArg batch, int nbatch, int nxs, int parts, int per_part, float reach_mult,
+    Vec3Arg centers, const float* __restrict__ coords, const float* __restrict__ types,
+    const float* __restrict__ radii, float4* __restrict__ slot_info, int* __restrict__ cand,
+    float4* __restrict__ records, int capacity) {
+  __shared__ int s_cnt[kSortWaves][kKeyGroup];   // atoms per (wave, key), then write positions
+  __shared__ int s_tot[kKeyGroup + 1];
+  __shared__ int s_rank, s_rmax, s_below;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int e = blockIdx.x / parts, part = blockIdx.x - e * parts;
+  const int c0 = part * per_part, c1 = min(g.ntypes, c0 + per_part);
+  const int nkeys = (c1 - c0) * nxs;
+  const int key_bits = 32 - __builtin_clz(max(nkeys - 1, 1));   // bits that tell the keys apart
+  const int kpad = (nkeys + kWave - 1) & ~(kWave - 1);          // keys the tables below cover
+  // the small loads first and together: this example's atoms, the size of one other example
+  // (for the rank below), the grid centre
+  const int32_t* const off = batch.offsets;
+  int begin = e * batch.per_example, end = begin + batch.per_example, first = 0, other_size = -1;
+  if (off != nullptr) {
+    first = off[0];
+    begin = off[e];
+    end = off[e + 1];
+    const int i = min(tid, nbatch - 1);
+    other_size = off[i + 1] - off[i];
+  }
+  const int n = max(end - begin, 0);
+  const int ntypes = g.ntypes;
+  const float radius_scale = g.radius_scale;
+  const float inv_slab = 0.25f / g.resolution;
+  const float3 center = load3(centers, e);
+  const float ox = center.x - g.half_dimension;
+  // every wave takes a contiguous run of whole 64-atom rounds, in atom order
+  const int per = ((n + kSortThreads - 1) / kSortThreads) * kWave;
+  const int wb = begin + wave * per, we = min(end, wb + per);
+  const bool cached = per <= kCached * kWave;
+
+  // key of an atom among this workgroup's; -1: a higher channel, -2: a lower one, -3: none
+  auto key_of = [&](float type, float x) -> int {
+    const float tf = floorf(type);
+    if (!(tf >= 0.f && tf < (float)ntypes)) return -3;
+    const int c = (int)tf;
+    if (c < c0) return -2;
+    if (c >= c1) return -1;
+    return (c - c0) * nxs + (int)slab_of(x, ox, inv_slab, nxs);
+  };
+
+  // the atoms of this thread, read once when they fit its registers
+  int c_key[kCached];
+  float c_x[kCached], c_y[kCached], c_z[kCached], c_r[kCached];
+  float my_rmax = 0.f;
+  int my_below = 0;
+  if (cached) {
+    // all loads first, unconditionally (a clamped atom number), so that they are in flight
+    // together; what they returned is looked at afterwards
+    float c_t[kCached];
+    const int last = max(end - 1, 0);
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) c_t[k] = c_x[k] = c_y[k] = c_z[k] = c_r[k] = 0.f;
+    if (n > 0) {                               // an example without atoms may come with no arrays
+#pragma unroll
+      for (int k = 0; k < kCached; ++k) {
+        const int ac = min(wb + k * kWave + lane, last);
+        c_t[k] = types[ac];
+        c_x[k] = coords[3 * ac];
+        c_y[k] = coords[3 * ac + 1];
+        c_z[k] = coords[3 * ac + 2];
+        c_r[k] = radii[ac];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) {
+      const bool have = n > 0 && wb + k * kWave + lane < we;
+      {
+#pragma clang fp contract(off)
+        c_r[k] = c_r[k] * radius_scale;
+      }
+      c_key[k] = have ? key_of(c_t[k], c_x[k]) : -3;
+      if (c_key[k] != -3) my_rmax = fmaxf(my_rmax, c_r[k]);
+      my_below += c_key[k] == -2 ? 1 : 0;
+    }
+  } else {
+    for (int a = wb + lane; a < we; a += kWave) {
+      const int key = key_of(types[a], coords[3 * a]);
+      if (key != -3) my_rmax = fmaxf(my_rmax, radii[a] * radius_scale);
+      my_below += key == -2 ? 1 : 0;
+    }
+  }
+
+  if (tid == 0) {
+    s_rank = 0;
+    s_rmax = 0;
+    s_below = 0;
+  }
+  for (int k = lane; k < kpad; k += kWave) s_cnt[wave][k] = 0;
+  __syncthreads();
+  // atoms of lower channels; the largest ar of the example; the rank of the example by size
+  // (descending, ties in input order)
+  // (reduced over the wave first: one LDS atomic per wave, not one per lane on one address)
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    my_below += __shfl_xor(my_below, d);
+    my_rmax = fmaxf(my_rmax, __shfl_xor(my_rmax, d));
+  }
+  if (lane == 0) {
+    if (my_below) atomicAdd(&s_below, my_below);
+    if (my_rmax > 0.f) atomicMax(&s_rmax, __float_as_int(my_rmax));   // positive floats order as ints
+  }
+  if (off != nullptr) {
+    int before = 0;
+    for (int i = tid; i < nbatch; i += kSortThreads) {
+      const int other = i == tid ? other_size : off[i + 1] - off[i];
+      before += (other > end - begin || (other == end - begin && i < e)) ? 1 : 0;
+    }
+    if (before) atomicAdd(&s_rank, before);
+  }
+  auto count = [&](int key) {
+    if (key >= 0) atomicAdd(&s_cnt[wave][key], 1);
+  };
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) count(c_key[k]);
+  } else {
+    for (int a = wb + lane; a < we; a += kWave) count(key_of(types[a], coords[3 * a]));
+  }
+  __syncthreads();
+  const int slot = off != nullptr ? s_rank : e;
+  if (tid == 0 && part == 0)
+    slot_info[slot] = make_float4(ox, center.y - g.half_dimension, center.z - g.half_dimension,
+                                  __int_as_float(e));
+  // how far in x the atoms of this example reach, at most (with a margin over the cull's slack)
+  const float reach = __int_as_float(s_rmax) * reach_mult * 1.0001f + 1e-3f;
+  const int base = begin - first + s_below;      // first record of this workgroup's channels
+
+  // per key: waves in order
+  for (int k = tid; k < kpad; k += kSortThreads) {
+    int run = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+      const int v = s_cnt[w][k];
+      s_cnt[w][k] = run;
+      run += v;
+    }
+    s_tot[k] = run;
+  }
+  __syncthreads();
+  // keys in order: every lane of wave 0 owns kpad / 64 consecutive keys
+  if (wave == 0) {
+    const int kper = kpad / kWave;
+    int sum = 0;
+    for (int j = 0; j < kper; ++j) sum += s_tot[lane * kper + j];
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int t = __shfl_up(incl, d);
+      if (lane >= d) incl += t;
+    }
+    int run = incl - sum;
+    for (int j = 0; j < kper; ++j) {
+      const int v = s_tot[lane * kper + j];
+      s_tot[lane * kper + j] = run;
+      run += v;
+    }
+    if (lane == kWave - 1) s_tot[kpad] = incl;
+  }
+  __syncthreads();
+  for (int k = lane; k < kpad; k += kWave) s_cnt[wave][k] += base + s_tot[k];
+  // per channel and x slab: the run of records whose atoms can reach the slab's x planes; slab_of
+  // is monotone, so an atom inside [low plane - reach, high plane + reach] has its slab in range.
+  // Keys past the last one hold no atoms, so their start is the end of the last.
+  int* const crow = cand + ((size_t)slot * ntypes + c0) * nxs * 2;
+  for (int i = tid; i < nkeys; i += kSortThreads) {
+    const int c = i / nxs, xs = i - c * nxs;
+    const float clx = grid_coord(ox, xs * kColXY, g.resolution);
+    const float chx = grid_coord(ox, min(xs * kColXY + kColXY, g.dim) - 1, g.resolution);
+    const int s_lo = (int)slab_of(clx - reach, ox, inv_slab, nxs);
+    const int s_hi = (int)slab_of(chx + reach, ox, inv_slab, nxs);
+    crow[2 * i] = base + s_tot[c * nxs + s_lo];
+    crow[2 * i + 1] = base + s_tot[c * nxs + s_hi + 1];
+  }
+  __syncthreads();
+  // scatter, in atom order within (wave, key): the lanes of a round that share a key take
+  // consecutive positions from the key's running position
+  auto scatter = [&](int key, float x, float y, float z, float ar) {
+    const bool act = key >= 0;
+    if (!act) key = 0;
+    unsigned long long same = __ballot(act);
+    if (same == 0) return;
+    for (int bit = 0; bit < key_bits; ++bit) {
+      const bool set = (key >> bit) & 1;
+      const unsigned long long bm = __ballot(act && set);
+      same &= set ? bm : ~bm;
+    }
+    const int leader = act ? (int)__builtin_ctzll(same) : lane;
+    int pos = 0;
+    if (act && lane == leader) pos = atomicAdd(&s_cnt[wave][key], (int)__popcll(same));
+    pos = __shfl(pos, leader);
+    if (act) {
+      pos += __popcll(same & ((1ull << lane) - 1ull));
+      if (pos < capacity) records[pos] = make_float4(x, y, z, ar);
+    }
+  };
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kCached; ++k)
+      if (wb + k * kWave < we)                 // uniform over the wave
+        scatter(c_key[k], c_x[k], c_y[k], c_z[k], c_r[k]);
+  } else {
+    for (int a0 = wb; a0 < we; a0 += kWave) {
+      const int a = a0 + lane;
+      const int ac = a < we ? a : we - 1;
+      const float x = coords[3 * ac];
+      float ar;
+      {
+#pragma clang fp contract(off)
+        ar = radii[ac] * radius_scale;
+      }
+      scatter(a < we ? key_of(types[ac], x) : -3, x, coords[3 * ac + 1], coords[3 * ac + 2], ar);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Launch 2
+// ------------------------------------------------------------------------------------------
+template <bool BINARY, bool EXACT, int COLS>
+__global__ __launch_bounds__(kWave) void splat_sorted_kernel(
+    GridArg g, const float4* __restrict__ slot_info, const int* __restrict__ cand,
+    const float4* __restrict__ records, int capacity, float* __restrict__ out,
+    int nxs, int nyp, int nzs, int nranges, int aligned_rows) {
+  __shared__ __align__(16) float stage[kPlane];
+
+  const int lane = threadIdx.x;
+  const int dim = g.dim;
+  const int ntypes = g.ntypes;
+  const size_t chan_stride = (size_t)dim * dim * dim;   // the host has checked: < 2^30 floats
+
+  // lane-constant part of the write-out of a column: the 192 float4 pieces of its 16 z rows in
+  // memory order (x, y, z), 64 at a time; the four rows of an x follow each other in memory
+  const int lx = lane >> 4, ly = (lane >> 2) & 3, lz = lane & 3;
+  const int stage_lane = (lx * 4 + ly) * kRowPad + lz;
+  int st_lds[kPieces], st_rx[kPieces], st_ry[kPieces], st_z[kPieces];
+  unsigned st_rel[kPieces];
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) {
+    const int p = lane + k * kWave;
+    const int r = p / 12, f4 = p - r * 12;
+    st_lds[k] = r * kRowPad + f4 * 4;
+    st_rx[k] = r >> 2;
+    st_ry[k] = r & 3;
+    st_z[k] = f4 * 4;
+    st_rel[k] = (unsigned)((st_rx[k] * dim + st_ry[k]) * dim + st_z[k]) * 4u;
+  }
+  float quad_c = g.C;
+  asm volatile("" : "+v"(quad_c));          // vector register (an fma takes one scalar operand)
+  const float frm2 = uniform(g.frm * g.frm);
+  const float grm2 = uniform(g.grm * g.grm);
+  const float inv_block = 0.25f / g.resolution;             // blocks per unit length along z
+  const __amdgpu_buffer_rsrc_t rec_buf = buffer_of(records, (size_t)capacity * 16);
+  auto load_round = [&](int first) -> v4u {
+    return __builtin_amdgcn_raw_buffer_load_b128(rec_buf, (first + lane) * 16, 0, 0);
+  };
+
+  // which item: channel range fastest, then the territory, then the example's slot
+  int t = blockIdx.x;
+  const int range = t % nranges;
+  t /= nranges;
+  const int yp = t % nyp;
+  t /= nyp;
+  const int zs = t % nzs;
+  t /= nzs;
+  const int xs = t % nxs;
+  const int slot = t / nxs;
+  const int nmine = (ntypes - range + nranges - 1) / nranges;   // channels range, range + R, ...
+  if (nmine <= 0) return;
+
+  const float4 info = slot_info[slot];
+  const int e = __builtin_amdgcn_readfirstlane(__float_as_int(info.w));
+  // first and one-past-last candidate record of this lane's channel
+  const __amdgpu_buffer_rsrc_t cand_buf =
+      buffer_of(cand + (size_t)slot * ntypes * nxs * 2, (size_t)ntypes * nxs * 8);
+  const int my_chan = range + lane * nranges;
+  v2u se = {0u, 0u};
+  if (lane < nmine) se = __builtin_amdgcn_raw_buffer_load_b64(cand_buf, (my_chan * nxs + xs) * 8, 0, 0);
+
+  const int x0 = xs * kColXY, y0 = yp * (kColXY * COLS), z0 = zs * kSlabZ;
+  const int zend = min(z0 + kSlabZ, dim);
+  float* const out_e = out + (size_t)e * ntypes * chan_stride;
+  const unsigned base_off = (unsigned)((x0 * dim + y0) * dim + z0) * 4u;
+
+  bool st_live[kPieces][COLS];
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k)
+#pragma unroll
+    for (int col = 0; col < COLS; ++col)
+      st_live[k][col] = x0 + st_rx[k] < dim && y0 + col * kColXY + st_ry[k] < dim && z0 + st_z[k] < zend;
+
+  // One column of one channel -> global memory as z rows, from the stage or as zeros.
+  auto store_column = [&](int c, int col, bool from_stage) {
+    const __amdgpu_buffer_rsrc_t out_buf = buffer_of(out_e + (size_t)c * chan_stride, chan_stride * 4);
+    const unsigned col_off = (unsigned)(col * kColXY * dim) * 4u;
+#pragma unroll
+    for (int k = 0; k < kPieces; ++k) {
+      if (st_live[k][col]) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (from_stage) v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
+        const unsigned off = base_off + col_off + st_rel[k];
+        if (aligned_rows && z0 + st_z[k] + 3 < dim) {
+          // non-temporal: nothing reads the grids back soon enough to find them in the
+          // last-level cache, and without the hint its write-back runs on into the next kernel
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf, (int)off, 0, 2);
+        } else {
+          const float ev[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (z0 + st_z[k] + j < dim)
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, ev[j]), out_buf,
+                                                    (int)(off + 4u * j), 0, 0);
+        }
+      }
+    }
+  };
+
+  unsigned long long full = __ballot(lane < nmine && se.y > se.x);    // my channels with atoms
+  unsigned long long empty = __ballot(lane < nmine && se.y <= se.x);  // and without
+  v4u pre = {0u, 0u, 0u, 0u};
+  if (full) pre = load_round(__builtin_amdgcn_readlane((int)se.x, (int)__builtin_ctzll(full)));
+
+  // ---- channels none of whose atoms can reach these x planes: zeros ----------------------------
+  while (empty != 0) {
+    const int j = __builtin_ctzll(empty);
+    empty &= empty - 1ull;
+#pragma unroll
+    for (int col = 0; col < COLS; ++col) store_column(range + j * nranges, col, false);
+  }
+  if (full == 0) return;
+
+  // ---- geometry of the territory -----------------------------------------------------------------
+  const float ox = uniform(info.x), oy = uniform(info.y), oz = uniform(info.z);
+  // first/last voxel centre of the territory inside the grid
+  const float clx = uniform(grid_coord(ox, x0, g.resolution));
+  const float chx = uniform(grid_coord(ox, min(x0 + kColXY, dim) - 1, g.resolution));
+  const float clz = uniform(grid_coord(oz, z0, g.resolution));
+  float cly[COLS], chy[COLS];
+  const int vxi = x0 + lx;
+  const float vx = grid_coord(ox, vxi, g.resolution);
+  // a voxel outside the grid sits at infinity, where no atom reaches it
+  float vy[COLS], vz[kBlocks];
+#pragma unroll
+  for (int col = 0; col < COLS; ++col) {
+    const int cy0 = y0 + col * kColXY;
+    cly[col] = uniform(grid_coord(oy, min(cy0, dim - 1), g.resolution));
+    chy[col] = uniform(grid_coord(oy, min(cy0 + kColXY, dim) - 1, g.resolution));
+    const int vyi = cy0 + ly;
+    vy[col] = (vxi < dim && vyi < dim) ? grid_coord(oy, vyi, g.resolution) : INFINITY;
+  }
+#pragma unroll
+  for (int q = 0; q < kBlocks; ++q) {
+    const int vzi = z0 + q * 4 + lz;
+    vz[q] = vzi < zend ? grid_coord(oz, vzi, g.resolution) : INFINITY;
+  }
+  const int last_block = (zend - z0 + 3) / 4 - 1;
+
+  // ---- channels with atoms ---------------------------------------------------------------------
+  while (full != 0) {
+    const int j = __builtin_ctzll(full);
+    full &= full - 1ull;
+    const int c = range + j * nranges;
+    const int lo = __builtin_amdgcn_readlane((int)se.x, j);
+    const int hi = __builtin_amdgcn_readlane((int)se.y, j);
+    // where the records of my next channel with atoms begin
+    const int next_lo = full ? __builtin_amdgcn_readlane((int)se.x, (int)__builtin_ctzll(full)) : lo;
+
+    float acc[COLS][kBlocks];
+#pragma unroll
+    for (int col = 0; col < COLS; ++col)
+#pragma unroll
+      for (int q = 0; q < kBlocks; ++q) acc[col][q] = 0.f;
+    unsigned touched = 0;                        // columns some record reaches
+
+    // A cull round takes 64 records, one per lane: for every column the lane finds the interval
+    // of z the atom can reach inside it (its reach shrunk by the distance to the column's
+    // footprint in x and y) and from it the range of blocks, as a bit mask.  The records that
+    // reach the territory are then taken one at a time, in record order, each over the blocks
+    // of its masks; record and masks come straight from the lane that tested it.
+    for (int r0 = lo; r0 < hi; r0 += kWave) {
+      const bool valid = r0 + lane < hi;
+      const v4u raw = pre;
+      pre = load_round(r0 + kWave < hi ? r0 + kWave : next_lo);   // in flight during this round
+      const float rec_x = __uint_as_float(raw.x), rec_y = __uint_as_float(raw.y);
+      const float rec_z = __uint_as_float(raw.z), rec_ar = __uint_as_float(raw.w);
+      float ar2;
+      {
+#pragma clang fp contract(off)
+        ar2 = rec_ar * rec_ar;
+      }
+      const float rec_w = BINARY ? ar2 : 1.0f / ar2;
+      // squared reach, with the slack that keeps the cull a superset of the exact test
+      const float reach2 = (BINARY ? ar2 : frm2 * ar2) * kCullSlack;
+      const float ex = fmaxf(fmaxf(clx - rec_x, rec_x - chx), 0.f);
+      unsigned mask[COLS];
+      unsigned any = 0;
+#pragma unroll
+      for (int col = 0; col < COLS; ++col) {
+        const float ey = fmaxf(fmaxf(cly[col] - rec_y, rec_y - chy[col]), 0.f);
+        const float rz2 = reach2 - (ex * ex + ey * ey);
+        mask[col] = 0;
+        if (valid && y0 + col * kColXY < dim && rz2 >= 0.f) {
+          const float rz = __builtin_amdgcn_sqrtf(rz2);
+          // block q holds the voxel centres clz + (4q .. 4q+3) * resolution
+          const float top = (rec_z + rz - clz) * inv_block + 1e-3f;
+          const float bottom = (rec_z - rz - clz) * inv_block - (0.75f + 1e-3f);
+          const int qhi = min((int)floorf(top), last_block), qlo = max((int)ceilf(bottom), 0);
+          if (qlo <= qhi) mask[col] = (2u << qhi) - (1u << qlo);
+        }
+        any |= mask[col];
+      }
+      uint3 clip = make_uint3(0, 0, 0);
+      if (EXACT) {
+        // index box of the CPU loops (src/grid_maker.cpp:181-189)
+        float densityrad;
+        {
+#pragma clang fp contract(off)
+          densityrad = rec_ar * g.frm;
+        }
+        int blo[3], bhi[3];
+        bounds_1d(ox, rec_x, densityrad, g.resolution, dim, blo[0], bhi[0]);
+        bounds_1d(oy, rec_y, densityrad, g.resolution, dim, blo[1], bhi[1]);
+        bounds_1d(oz, rec_z, densityrad, g.resolution, dim, blo[2], bhi[2]);
+        clip = make_uint3((unsigned)blo[0] | ((unsigned)bhi[0] << 16),
+                          (unsigned)blo[1] | ((unsigned)bhi[1] << 16),
+                          (unsigned)blo[2] | ((unsigned)bhi[2] << 16));
+      }
+
+      unsigned long long todo = __ballot(any != 0);
+#pragma unroll 1
+      while (todo != 0) {                        // loses a bit per trip
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1ull;
+        const float rx = lane_value(rec_x, src), ry = lane_value(rec_y, src);
+        const float rz = lane_value(rec_z, src), rw = lane_value(rec_w, src);
+        float rar = 0.f;
+        uint3 rclip = make_uint3(0, 0, 0);
+        if (EXACT) {
+          rar = lane_value(rec_ar, src);
+          rclip = make_uint3((unsigned)__builtin_amdgcn_readlane((int)clip.x, src),
+                             (unsigned)__builtin_amdgcn_readlane((int)clip.y, src),
+                             (unsigned)__builtin_amdgcn_readlane((int)clip.z, src));
+        }
+        const float dx = vx - rx;
+#pragma unroll
+        for (int col = 0; col < COLS; ++col) {
+          const unsigned reach = (unsigned)__builtin_amdgcn_readlane((int)mask[col], src);
+          if (reach == 0) continue;
+          touched |= 1u << col;
+          const float dy = vy[col] - ry;
+          float dxy2;
+          if (BINARY) {
+#pragma clang fp contract(off)
+            dxy2 = dx * dx + dy * dy;
+          } else {
+            dxy2 = fmaf(dx, dx, dy * dy);
+          }
+#pragma unroll
+          for (int q0 = 0; q0 < kBlocks; q0 += 4) {
+            if (((reach >> q0) & 0xfu) == 0) continue;
+#pragma unroll
+            for (int q = q0; q < q0 + 4; ++q) {
+              if (((reach >> q) & 1u) == 0) continue;
+              const float dz = vz[q] - rz;
+              if (EXACT) {
+                float val;
+                const bool inside = inside_clip(vxi, y0 + col * kColXY + ly, z0 + q * 4 + lz, rclip);
+                const bool hit = density_hit<BINARY, true>(g, dx, dy, dz, rw, rar, frm2, grm2,
+                                                           quad_c, val);
+                if (hit && inside) acc[col][q] = BINARY ? 1.0f : acc[col][q] + val;
+              } else if (BINARY) {
+                float rsq;
+                {
+#pragma clang fp contract(off)
+                  rsq = dxy2 + dz * dz;
+                }
+                if (rsq < rw) acc[col][q] = 1.0f;
+              } else {
+                const float u = fmaf(dz, dz, dxy2) * rw;
+                if (u <= frm2) {
+                  const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                  const float su = __builtin_amdgcn_sqrtf(u);
+                  const float quad = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+                  acc[col][q] += (u <= grm2) ? gauss : quad;
+                }
+              }
+            }
+          }
+        }
+      }
+    }
+
+    // write-out, column by column: sums -> the stage -> z rows (or zeros straight away); LDS
+    // keeps the order of one wave's accesses, so no barrier is involved
+#pragma unroll
+    for (int col = 0; col < COLS; ++col) {
+      if (y0 + col * kColXY >= dim) break;
+      const bool from_stage = (touched >> col) & 1u;
+      if (from_stage) {
+#pragma unroll
+        for (int q = 0; q < kBlocks; ++q) stage[stage_lane + q * 4] = acc[col][q];
+      }
+      store_column(c, col, from_stage);
+    }
+  }
+}
+
+int exp_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
+
+template <bool BINARY, bool EXACT, int COLS>
+hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, float* out,
+                        hipStream_t stream) {
+  const int dim = g.dim;
+  const int nxs = (dim + kColXY - 1) / kColXY;
+  const int nyp = (dim + kColXY * COLS - 1) / (kColXY * COLS);
+  const int nzs = (dim + kSlabZ - 1) / kSlabZ;
+  static const int exp_ranges = exp_int("MOLGRID_EXP_RANGES", 0);
+  int nranges = std::max((g.ntypes + kItemChannels - 1) / kItemChannels,
+                         (g.ntypes + kItemChannelsMax - 1) / kItemChannelsMax);
+  if (exp_ranges) nranges = std::max(exp_ranges, (g.ntypes + kItemChannelsMax - 1) / kItemChannelsMax);
+  const long long nitems = (long long)nbatch * nxs * nzs * nyp * nranges;
+  if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
+  const int aligned = ((dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
+  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS>), dim3((unsigned)nitems), dim3(kWave),
+                     0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out, nxs, nyp, nzs,
+                     nranges, aligned);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+size_t forward_sorted_workspace_bytes(int nbatch, int atoms_per_example, int ntypes, int dim) {
+  const long long capacity = (long long)nbatch * atoms_per_example;
+  const size_t nkeys = (size_t)ntypes * ((dim + kColXY - 1) / kColXY);
+  return align256((size_t)nbatch * 16) + align256((size_t)nbatch * nkeys * 8) +
+         (size_t)capacity * 16;
+}
+
+// hipErrorInvalidValue = the case is not covered (a channel of 4 GB or more, more records than a
+// buffer addresses, a workspace that is too small).
+hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 const Vec3Arg& centers, const float* coords,
+                                 const float* type_index, const float* radii, float* out,
+                                 bool binary, bool exact, void* workspace, size_t workspace_bytes,
+                                 hipStream_t stream) {
+  const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
+  if (chan_stride * 4 >= 0xfffffff0ull) return hipErrorInvalidValue;
+  const long long capacity = (long long)nbatch * batch.per_example;
+  if (capacity * 16 >= 0xfffffff0ll) return hipErrorInvalidValue;
+  if (workspace == nullptr ||
+      workspace_bytes < forward_sorted_workspace_bytes(nbatch, batch.per_example, g.ntypes, g.dim))
+    return hipErrorInvalidValue;
+  const int nxs = (g.dim + kColXY - 1) / kColXY;
+  if ((long long)g.ntypes * nxs >= (1 << 26)) return hipErrorInvalidValue;
+  const SortedAtoms s = carve(workspace, nbatch, g.ntypes * nxs, capacity);
+  // channels per workgroup of the sort: a few, and no more keys than it handles
+  const int per_part = std::max(1, std::min(kItemChannels, kKeyGroup / nxs));
+  const int parts = (g.ntypes + per_part - 1) / per_part;
+  hipLaunchKernelGGL(sort_atoms_kernel, dim3((unsigned)(parts * nbatch)), dim3(kSortThreads), 0, stream, g,
+                     batch, nbatch, nxs, parts, per_part, binary ? 1.0f : g.frm, centers, coords,
+                     type_index, radii, s.slot_info, s.cand, s.records, s.capacity);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+
+  static const int cols = exp_int("MOLGRID_EXP_MODE", 0) & 3;          // 0: two columns, 1: one
+  if (exact) {
+    if (binary) return launch_splat<true, true, 1>(g, s, nbatch, out, stream);
+    return launch_splat<false, true, 1>(g, s, nbatch, out, stream);
+  }
+  if (binary) return launch_splat<true, false, 2>(g, s, nbatch, out, stream);
+  if (cols == 1) return launch_splat<false, false, 1>(g, s, nbatch, out, stream);
+  return launch_splat<false, false, 2>(g, s, nbatch, out, stream);
+}
+
+}  // namespace mg

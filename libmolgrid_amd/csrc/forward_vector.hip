@@ -263,16 +263,11 @@ hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nb
                                  const float* type_vector, const float* radii, float* out,
                                  bool binary, bool radii_type_indexed, bool exact,
                                  hipStream_t stream) {
-  // per-atom radii take the column kernel; type-indexed radii and the exact-predicate modes
+  // per-atom radii take the matrix-core kernel; type-indexed radii and the exact-predicate modes
   // (truncated Gaussian) use the cubic-tile kernel below
-  // (the matrix-core kernel; MOLGRID_HIP_VECTOR_COLUMN_KERNEL=1 keeps the column kernel)
-  const char* column_only = getenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL");
-  if (!radii_type_indexed && !exact && !(column_only != nullptr && column_only[0] == '1'))
+  if (!radii_type_indexed && !exact)
     return launch_forward_vector_mfma(g, batch, nbatch, centers, coords, type_vector, radii, out,
                                       binary, stream);
-  if (!radii_type_indexed && !exact)
-    return launch_forward_vector_column(g, batch, nbatch, centers, coords, type_vector, radii, out,
-                                        binary, exact, stream);
   if (binary && radii_type_indexed)
     return launch_sized<true, true>(g, batch, nbatch, centers, coords, type_vector, radii, out, exact, stream);
   if (binary)

@@ -26,22 +26,16 @@ hipError_t launch_transform(const BatchArg& batch, int nbatch, int launch_atoms,
                             const Vec3Arg& translations, bool dotranslate, bool inverse,
                             const float* in, float* out, hipStream_t stream);
 
-hipError_t launch_forward_index(const GridArg& g, const BatchArg& batch, int nbatch,
-                                const Vec3Arg& centers, const float* coords,
-                                const float* type_index, const float* radii, float* out,
-                                bool binary, bool exact, hipStream_t stream);
-
-// index types, one channel at a time (forward_channel.hip); hipErrorInvalidValue = not covered
-hipError_t launch_forward_channel(const GridArg& g, const BatchArg& batch, int nbatch,
-                                  const Vec3Arg& centers, const float* coords,
-                                  const float* type_index, const float* radii, float* out,
-                                  bool binary, hipStream_t stream);
-
-// vector types with per-atom radii: the column kernel of forward_index.hip
-hipError_t launch_forward_vector_column(const GridArg& g, const BatchArg& batch, int nbatch,
-                                        const Vec3Arg& centers, const float* coords,
-                                        const float* type_vector, const float* radii, float* out,
-                                        bool binary, bool exact, hipStream_t stream);
+// GridMaker::forward, index types, through sorted atom records (forward_sorted.hip): two launches,
+// a workspace of forward_sorted_workspace_bytes() in device memory.  hipErrorInvalidValue = the
+// case is not covered (a channel of 4 GB or more, more than 2^28 atom slots) or the workspace is
+// too small.
+size_t forward_sorted_workspace_bytes(int nbatch, int atoms_per_example, int ntypes, int dim);
+hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 const Vec3Arg& centers, const float* coords,
+                                 const float* type_index, const float* radii, float* out,
+                                 bool binary, bool exact, void* workspace, size_t workspace_bytes,
+                                 hipStream_t stream);
 
 // vector types with per-atom radii, density mode, on the matrix cores (forward_vector_mfma.hip)
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,

@@ -294,6 +294,7 @@ class AtomBatch(object):
         self.largest = max(int(np.max(np.diff(host))) if host.size > 1 else 0, 1)
         self.total = int(host[-1])
         self._dev = None
+        self.scratch = {}            # device workspaces that calls on this layout keep
 
     @property
     def dev(self):
@@ -1024,6 +1025,23 @@ class GridMaker(object):
                 raise IndexError("Type index %d larger than allowed %d"
                                  % (int(np.floor(t).max()), ntypes))
 
+    def _forward_index_call(self, batch=None):
+        """mg_forward_index_ws with a workspace from torch's allocator (which is stream aware); a
+        ragged batch layout (AtomBatch) keeps its workspace for the next call."""
+        def call(p, B, off, n, cen, chost, coords, types, radii, T, out, stream):
+            need = int(_lib.mg_forward_index_workspace_size(p, B, n, T))
+            ws = None
+            if need:
+                key = ("forward_index_ws", torch.cuda.current_device())
+                ws = batch.scratch.get(key) if batch is not None else None
+                if ws is None or ws.numel() < need:
+                    ws = torch.empty(need, dtype=torch.uint8, device=_device())
+                    if batch is not None:
+                        batch.scratch[key] = ws
+            return _lib.mg_forward_index_ws(p, B, off, n, cen, chost, coords, types, radii, T, out,
+                                            ws.data_ptr() if ws is not None else None, need, stream)
+        return call
+
     # -- forward ------------------------------------------------------------
     @_accepts_grids
     def forward(self, *args, **kw):
@@ -1078,7 +1096,7 @@ class GridMaker(object):
             if self._p.radii_type_indexed:
                 raise ValueError("Type indexed radii not supported with index types.")
             self._check_host_types(types, a_out.shape[0])
-            fn = _lib.mg_forward_index
+            fn = self._forward_index_call()
         else:
             self._check_vector_args(n, a_types, a_radii, a_out.shape)
             fn = _lib.mg_forward_vector
@@ -1169,7 +1187,7 @@ class GridMaker(object):
             if self._p.radii_type_indexed:
                 raise ValueError("Type indexed radii not supported with index types.")
             self._check_host_types(types, a_out.shape[1])
-            fn = _lib.mg_forward_index
+            fn = self._forward_index_call()
         else:
             self._check_vector_args(n, _Shape(a_types.shape[1:]), _Shape(a_radii.shape[1:]),
                                     a_out.shape[1:])
@@ -1204,7 +1222,7 @@ class GridMaker(object):
             if a_radii.shape[0] < total:
                 raise IndexError("radii does not match number of atoms")
             self._check_host_types(types, T)
-            fn = _lib.mg_forward_index
+            fn = self._forward_index_call(offsets if isinstance(offsets, AtomBatch) else None)
         else:
             if a_types.shape[1] != T:
                 raise IndexError("number of types in type_vector does not match number of "

@@ -99,7 +99,7 @@ def test_many_atoms_on_one_spot(mg):
     ref = oracle.GridMaker(0.5, 7.5).forward((0, 0, 0), coords, types, radii, 2)
     got = gpu_forward(mg, (0.5, 7.5), (0, 0, 0), coords, types, radii, 2)
     # thousands of terms per voxel: same summation order, so still tight
-    assert_close(got, ref, rtol=2e-5, what="dense forward")
+    assert_close(got, ref, what="dense forward")
 
 
 def test_empty_and_ignored_atoms(mg):
@@ -193,7 +193,7 @@ def test_repeat_runs_are_bit_identical(mg):
 
 
 def test_more_channels_than_the_channel_sort_handles(mg):
-    """70 channels: every channel scans the atoms again instead of one sort (any channel count)."""
+    """70 channels: more than one wave's worth of channels per territory at the default split."""
     rng = np.random.default_rng(70)
     coords, types, radii = synth.small_index_case(rng, 400, 70, 8.0)
     for binary in (False, True):
@@ -205,28 +205,48 @@ def test_more_channels_than_the_channel_sort_handles(mg):
             assert_close(got, ref, what="70 channels")
 
 
-def test_column_kernel_gives_the_same_values(mg, monkeypatch):
-    """The second implementation of the index-type forward pass (one column of all channels per
-    pass) sums in the same order: identical grids, dense and binary, also for a ragged batch."""
+def test_library_workspace_and_callers_workspace_give_the_same_grid(mg):
+    """mg_forward_index (workspace kept by the library, grown on demand) and mg_forward_index_ws
+    (workspace passed in) run the same launches: identical grids, dense and binary, for a small
+    call followed by a larger one (the library's workspace grows) and a small one again."""
+    import ctypes
+    from libmolgrid_amd import _capi
+    lib = _capi.lib
     rng = np.random.default_rng(5)
-    coords, types, radii = synth.small_index_case(rng, 900, 28, 14.0)
-    for binary in (False, True):
-        monkeypatch.delenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL", raising=False)
-        a = gpu_forward(mg, (0.5, 23.5, binary), (0.3, -0.2, 0.1), coords, types, radii, 28)
-        monkeypatch.setenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL", "1")
-        b = gpu_forward(mg, (0.5, 23.5, binary), (0.3, -0.2, 0.1), coords, types, radii, 28)
-        monkeypatch.delenv("MOLGRID_HIP_FORWARD_COLUMN_KERNEL")
-        assert np.array_equal(a, b)
-        ref = oracle.GridMaker(0.5, 23.5, binary).forward((0.3, -0.2, 0.1), coords, types, radii, 28)
-        if binary:
-            assert np.array_equal(b, ref)
-        else:
-            assert_close(b, ref, what="column kernel")
+    for natoms in (40, 900, 60):
+        coords, types, radii = synth.small_index_case(rng, natoms, 28, 14.0)
+        dc, dt, dr = dev(coords), dev(types), dev(radii)
+        for binary in (False, True):
+            gm = mg.GridMaker(0.5, 23.5, binary)
+            shape = gm.grid_dimensions(28)
+            a = torch.full(shape, 3.0, device="cuda")
+            b = torch.full(shape, 5.0, device="cuda")
+            center = _capi.f3((0.3, -0.2, 0.1))
+            need = lib.mg_forward_index_workspace_size(gm._p, 1, natoms, 28)
+            assert need > 0
+            ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            stream = torch.cuda.current_stream().cuda_stream
+            assert lib.mg_forward_index_ws(gm._p, 1, None, natoms, None, center, dc.data_ptr(),
+                                           dt.data_ptr(), dr.data_ptr(), 28, a.data_ptr(),
+                                           ws.data_ptr(), need, stream) == 0
+            assert lib.mg_forward_index(gm._p, 1, None, natoms, None, center, dc.data_ptr(),
+                                        dt.data_ptr(), dr.data_ptr(), 28, b.data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(a, b)
+            ref = oracle.GridMaker(0.5, 23.5, binary).forward((0.3, -0.2, 0.1), coords, types, radii, 28)
+            if binary:
+                assert np.array_equal(b.cpu().numpy(), ref)
+            else:
+                assert_close(b.cpu().numpy(), ref, what="library workspace")
+            # a workspace that is too small is refused, nothing is launched
+            assert lib.mg_forward_index_ws(gm._p, 1, None, natoms, None, center, dc.data_ptr(),
+                                           dt.data_ptr(), dr.data_ptr(), 28, a.data_ptr(),
+                                           ws.data_ptr(), need - 1, stream) == _capi.MG_ERR_INVALID_ARGUMENT
 
 
 def test_more_atoms_than_sixteen_bit_indices(mg):
-    """70,000 atoms in one example (survivor lists hold 16-bit atom numbers: the atoms are then
-    taken in passes), most of them far from the grid; dense and binary."""
+    """70,000 atoms in one example (more than the sort keeps in registers: it then reads the
+    atoms once per pass), most of them far from the grid; dense and binary."""
     rng = np.random.default_rng(77)
     coords, types, radii = synth.small_index_case(rng, 70000, 4, 30.0)
     for binary in (False, True):

@@ -95,11 +95,10 @@ def test_backward_full_batch(mg, workload):
     assert torch.equal(grads2, grads * 2)
 
 
-def test_vector_types_full_size_properties(mg, monkeypatch):
+def test_vector_types_full_size_properties(mg):
     """Configuration 3 at its full size (16 x 10,000 atoms into 28x96^3) without the oracle: the
-    grid is linear in the type vectors, one example of the batch equals its single launch, the
-    matrix-core kernel agrees with the column kernel, and a one-hot type vector gives the
-    index-typed grid."""
+    grid is linear in the type vectors, one example of the batch equals its single launch, and a
+    one-hot type vector gives the index-typed grid."""
     v = synth.vector_batch()
     B = len(v["offsets"]) - 1
     gm = mg.GridMaker(0.25, 23.75)
@@ -129,24 +128,6 @@ def test_vector_types_full_size_properties(mg, monkeypatch):
     one = torch.empty(dims, device="cuda")
     gm.forward(tuple(v["centers"][9]), coords[s], w[s], radii[s], one)
     assert torch.equal(one, full[9])
-    # the column kernel sums in atom order, the matrix cores four atoms at a time
-    monkeypatch.setenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", "1")
-    col = grid(w, slice(12, 14))
-    monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
-    err = (col - full[12:14]).abs()
-    assert float((err - 1e-5 * col.abs()).max()) <= 1e-6
-    # binary occupancy (sums of weights, about 35 per voxel): the two kernels agree bit for bit
-    gmb = mg.GridMaker(0.25, 23.75, True)
-    n0, n1 = int(off[12]), int(off[14])
-    bin_mfma = torch.empty((2,) + dims, device="cuda")
-    gmb.forward_batch(off[12:15] - off[12], v["centers"][12:14], coords[n0:n1], w[n0:n1],
-                      radii[n0:n1], bin_mfma)
-    monkeypatch.setenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL", "1")
-    bin_col = torch.empty((2,) + dims, device="cuda")
-    gmb.forward_batch(off[12:15] - off[12], v["centers"][12:14], coords[n0:n1], w[n0:n1],
-                      radii[n0:n1], bin_col)
-    monkeypatch.delenv("MOLGRID_HIP_VECTOR_COLUMN_KERNEL")
-    assert torch.equal(bin_mfma, bin_col) and float(bin_col.max()) > 1.0
     # one-hot weights: the index-typed grid
     types = torch.randint(0, 28, (int(off[1]),), device="cuda")
     hot = torch.zeros((int(off[1]), 28), device="cuda")
@@ -157,6 +138,26 @@ def test_vector_types_full_size_properties(mg, monkeypatch):
     gm.forward(tuple(v["centers"][0]), coords[:int(off[1])], types.float(), radii[:int(off[1])], b)
     err = (a - b).abs()
     assert float((err - 1e-5 * b.abs()).max()) <= 1e-6
+
+
+@pytest.mark.parametrize("binary", [False, True])
+def test_vector_types_full_size_example_vs_oracle(mg, binary):
+    """One whole example of configuration 3 (10,000 atoms, 28 soft types, 28x96^3) against the CPU
+    loop (src/grid_maker.cpp:214-271): densities within 1e-6 + 1e-5*|ref|, binary occupancy (sums
+    of about 35 weights per voxel, added four atoms per matrix-core step) bit for bit."""
+    v = synth.vector_batch(nbatch=1, natoms=10000)
+    ref = oracle.GridMaker(0.25, 23.75, binary).forward_batch(
+        v["offsets"], v["centers"], v["coords"], v["types"], v["radii"], 28, nthreads=8)
+    gm = mg.GridMaker(0.25, 23.75, binary)
+    out = torch.empty((1,) + gm.grid_dimensions(28), device="cuda")
+    gm.forward_batch(v["offsets"], v["centers"], dev(v["coords"]), dev(v["types"]),
+                     dev(v["radii"]), out)
+    got = out.cpu().numpy()
+    if binary:
+        assert float(ref.max()) > 1.0
+        assert np.array_equal(got, ref)
+    else:
+        assert_close(got, ref, what="config 3, full example")
 
 
 def test_interpolation_full_size_properties(mg):
