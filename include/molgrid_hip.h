@@ -130,6 +130,21 @@ int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offs
                      const float* type_index, const float* radii, int ntypes, float* out,
                      void* stream);
 
+/* No counterpart in the reference.  mg_forward_index for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops, harnesses
+ * that forbid hipMalloc): the workspace is a fixed array of
+ * MG_STATIC_SCRATCH_BYTES in the library's device code, one copy per GPU, held
+ * until the process ends.  Nothing is allocated or freed.  Sizes whose workspace
+ * (mg_forward_index_workspace_size) exceeds the array return MG_ERR_OUT_OF_RANGE
+ * and launch nothing.  Every call on a GPU uses that GPU's one array: calls that
+ * overlap on one GPU (different streams) race. */
+#define MG_STATIC_SCRATCH_BYTES (16u << 20)
+int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                            int atoms_per_example, const float* grid_centers,
+                            const float grid_center_host[3], const float* coords,
+                            const float* type_index, const float* radii, int ntypes, float* out,
+                            void* stream);
+
 /* GridMaker::forward, vector types; replaces forward_gpu_vec and its launcher
  * (src/grid_maker.cu:348-441), values of src/grid_maker.cpp:214-271.
  *   type_vector [n, ntypes]; radii [n], or [nbatch, ntypes] when

@@ -14,11 +14,12 @@ MG_ERR_INVALID_ARGUMENT = -1
 MG_ERR_OUT_OF_RANGE = -2
 MG_ERR_UNSUPPORTED = -3
 MG_ERR_NULL_POINTER = -4
+MG_STATIC_SCRATCH_BYTES = 16 << 20
 
 EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
-    "mg_forward_index_workspace_size", "mg_forward_vector", "mg_backward_index",
+    "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_vector", "mg_backward_index",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate",
 )
 
@@ -64,6 +65,7 @@ def _load():
     lib.mg_transform_backward.argtypes = tr
     fwd = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp]
     lib.mg_forward_index.argtypes = fwd
+    lib.mg_forward_index_static.argtypes = fwd
     lib.mg_forward_index_ws.argtypes = fwd[:-1] + [_vp, ctypes.c_size_t, _vp]
     lib.mg_forward_index_workspace_size.argtypes = [gm, _i, _i, _i]
     lib.mg_forward_index_workspace_size.restype = ctypes.c_size_t

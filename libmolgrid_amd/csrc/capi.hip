@@ -8,6 +8,11 @@
 #include "kernels.h"
 #include "molgrid_hip.h"
 
+// Scratch memory of mg_forward_index_static, part of the loaded code object: every GPU the library
+// runs on holds its own copy at its own address until the process ends.  Host code never uses the
+// array's name as an address; it asks for the device address once per device (static_scratch()).
+static __device__ __align__(256) unsigned char scratch[MG_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 using namespace mg;
@@ -256,6 +261,53 @@ int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offs
   return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
                             grid_center_host, coords, type_index, radii, ntypes, out, workspace, bytes,
                             stream);
+}
+
+namespace {
+
+void* g_scratch_address[kMaxDevices] = {nullptr};   // device address of `scratch`, per device
+std::mutex g_scratch_mutex;
+
+// Device address of the current device's copy of `scratch` (asked for on the first call on that
+// device); the error of the lookup otherwise.
+hipError_t static_scratch(void** address) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_address[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_address[dev] = p;
+  }
+  *address = g_scratch_address[dev];
+  return hipSuccess;
+}
+
+}  // namespace
+
+int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                            int atoms_per_example, const float* grid_centers,
+                            const float grid_center_host[3], const float* coords,
+                            const float* type_index, const float* radii, int ntypes, float* out,
+                            void* stream) {
+  bool nothing = false;
+  const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
+                                    radii, ntypes, out, &nothing);
+  if (s != MG_OK || nothing) return s;
+  if (mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes) > MG_STATIC_SCRATCH_BYTES)
+    return MG_ERR_OUT_OF_RANGE;
+  void* address = nullptr;
+  const hipError_t e = static_scratch(&address);
+  if (e != hipSuccess) return from_hip(e);
+  // nothing in the scratch has to start at zero: the sort launch writes every table entry and
+  // every record that the splat launch reads
+  return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
+                            grid_center_host, coords, type_index, radii, ntypes, out, address,
+                            MG_STATIC_SCRATCH_BYTES, stream);
 }
 
 int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
