@@ -24,12 +24,14 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 
-def event_ms(fn, iters):
-    """Average milliseconds of fn() over iters launches, timed with events on the
-    stream the kernels are launched on (torch's current stream)."""
+def event_ms(fn, iters, warmup=2):
+    """Average milliseconds of fn() over iters launches after `warmup` untimed ones, timed with
+    events on the stream the kernels are launched on (torch's current stream)."""
     import torch
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
+    for _ in range(warmup):
+        fn()
     torch.cuda.synchronize()
     start.record()
     for _ in range(iters):
@@ -58,11 +60,15 @@ def step_breakdown(fns, iters):
             for i in range(len(fns))]
 
 
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_step_config1_kernel_trace.txt")
+
+
 def measured_traffic(kernel):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary
-    (FETCH_SIZE + WRITE_SIZE, KiB per dispatch; calibration factor 1.0, stated in that file).
-    None when the summary is missing or does not list the kernel."""
-    path = os.path.join(ROOT, "profiles", "bench_step_config1_kernel_trace.txt")
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary of this same
+    command (FETCH_SIZE + WRITE_SIZE, KiB per dispatch; calibration factor 1.0, stated in that
+    file) -- counters cannot be read from inside the run, so this figure is only as fresh as that
+    file.  None when the summary is missing or does not list the kernel."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
     try:
         lines = open(path).read().splitlines()
     except OSError:
@@ -102,8 +108,42 @@ def cpu_baseline(cfg, ntypes, nsample, threads):
     return dict(total_s=t2 - t0, forward_s=t1 - t0, backward_s=t2 - t1, atoms=n)
 
 
-def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, diff, grads, n_atoms,
-                    bwd_bytes):
+def parity_sample(cfg, gm_args, ntypes, nsample, moved, grid, diff, grads):
+    """Distance of the step's results from the CPU oracle on the first `nsample` examples: max
+    abs error, max relative error and the number of values outside 1e-6 + 1e-5*|ref|; the atom
+    gradients against the oracle's sums in double and against its float loop (the reference's
+    order), whose own distance from the sums in double is given beside them."""
+    import oracle
+    from util import parity_stats
+    off = cfg["offsets"][: nsample + 1]
+    n = int(off[-1])
+    og = oracle.GridMaker(*gm_args)
+    m = moved[:n].cpu().numpy()
+    ref_moved = oracle.transform_forward_batch(off, cfg["quats"], cfg["centers"],
+                                               cfg["translations"], cfg["coords"][:n], nthreads=8)
+    ref_grid = og.forward_batch(off, cfg["centers"], ref_moved, cfg["types"][:n], cfg["radii"][:n],
+                                ntypes, nthreads=8)
+    d = diff[:nsample].cpu().numpy()
+    g32 = og.backward_batch(off, cfg["centers"], ref_moved, cfg["types"][:n], cfg["radii"][:n], d,
+                            nthreads=8)
+    g64 = np.concatenate([og.backward(cfg["centers"][b], ref_moved[off[b]:off[b + 1]],
+                                      cfg["types"][off[b]:off[b + 1]],
+                                      cfg["radii"][off[b]:off[b + 1]], d[b], f64=True)
+                          for b in range(nsample)])
+    got_g = grads[:n].cpu().numpy()
+    return {
+        "sample": "first %d examples (%d atoms) against the CPU oracle" % (nsample, n),
+        "tolerance": "1e-6 + 1e-5*|ref|",
+        "transform_bit_exact": bool(np.array_equal(m, ref_moved)),
+        "forward": parity_stats(grid[:nsample].cpu().numpy(), ref_grid),
+        "backward_vs_f64_sums": parity_stats(got_g, g64),
+        "backward_vs_float_loop": parity_stats(got_g, g32),
+        "float_loop_vs_f64_sums": parity_stats(g32, g64),
+    }
+
+
+def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, diff, grads,
+                    n_atoms, bwd_bytes):
     """The remaining configurations, one kernel each, events on the launch stream: the backward
     pass with 90 % of the upstream gradient zeroed (configuration 2), vector types into 28x96^3
     for Gaussian and binary density (configuration 3), trilinear resampling under random rotations
@@ -124,18 +164,25 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, diff, 
     res["backward_sparse10"] = entry(ms, bwd_bytes,
                                      atom_grads_per_s=round(n_atoms / (ms * 1e-3), 1))
 
-    # configuration 4: resample 50 x 28 x 48^3 under per-example rotations and +-1.5 A shifts
-    B, K, D = diff.shape[0], diff.shape[1], diff.shape[2]
+    # configuration 4: the gridded configuration-1 atoms with N(0, 0.1) noise on 5 % of the
+    # voxels, resampled under per-example rotations and +-1.5 A shifts
+    B, K, D = grid.shape[0], grid.shape[1], grid.shape[2]
+    gm.forward_batch(offsets, centers, moved, types, radii, grid)
+    src = diff                                   # reuse the buffer of the upstream gradient
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    src.normal_(0.0, 0.1, generator=gen)
+    src.mul_((torch.rand(src.shape, device="cuda", generator=gen) < 0.05).to(src.dtype))
+    src.add_(grid)
     rng = np.random.default_rng(4)
     quats = torch.as_tensor(synth.random_quaternions(rng, B)).cuda()
     shifts = torch.as_tensor(rng.uniform(-1.5, 1.5, (B, 3)).astype(np.float32)).cuda()
     zeros = torch.zeros((B, 3), device="cuda")
-    dst = torch.empty_like(diff)
+    dst = grid                                   # the forward pass's output buffer
     gi = mg.GridInterpolater(0.5, 23.5, 0.5, 23.5)
-    ms = event_ms(lambda: gi.forward_batch(diff, quats, zeros, shifts, dst), 10)
-    res["interpolate"] = entry(ms, 2 * diff.numel() * 4, grids_per_s=round(B / (ms * 1e-3), 1),
-                               workload="configs[4]: %d x %dx%d^3, random rotation, +-1.5 A" % (B, K, D))
-    del dst
+    ms = event_ms(lambda: gi.forward_batch(src, quats, zeros, shifts, dst), 10)
+    res["interpolate"] = entry(ms, 2 * src.numel() * 4, grids_per_s=round(B / (ms * 1e-3), 1),
+                               workload="configs[4]: %d x %dx%d^3 gridded atoms + 5 %% noise, "
+                                        "random rotation, +-1.5 A" % (B, K, D))
 
     # configuration 3: 16 x 10,000 atoms with 28-float type vectors into 28x96^3
     v = synth.vector_batch(nbatch=16, natoms=10000)
@@ -267,14 +314,17 @@ def main():
 
     dominant_fwd = ms_fwd >= ms_bwd
     roofline = {
-        "kernel": "splat_channel_kernel (forward)" if dominant_fwd else "backward_index_kernel",
+        # one forward call = sort_atoms_kernel + splat_sorted_kernel; the duration is that of both
+        "kernel": "sort_atoms_kernel + splat_sorted_kernel (forward)" if dominant_fwd
+                  else "backward_index_kernel",
         "bound": "hbm",
         "achieved": round(fwd_gbs if dominant_fwd else bwd_gbs, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
-        "traffic": measured_traffic("splat_channel_kernel" if dominant_fwd
+        "traffic": measured_traffic("splat_sorted_kernel" if dominant_fwd
                                     else "backward_index_kernel"),
+        "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 counters of this command, not of this run)",
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
         # the same kernel between the other launches of the step (see step_breakdown)
@@ -292,9 +342,18 @@ def main():
                       "unrotate_in_step_ms": round(in_step[3], 4)},
     }
 
+    parity = None
+    if not args.no_cpu:
+        # the step once more, gradients before their un-rotation, against the oracle
+        k_transform()
+        k_forward()
+        k_backward()
+        torch.cuda.synchronize()
+        parity = parity_sample(cfg, (0.5, 23.5), T, min(B, 5), moved, grid, diff, grads)
+
     if not args.no_extras:
-        kernels.update(other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, diff,
-                                       grads, n_atoms, bwd_bytes))
+        kernels.update(other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid,
+                                       diff, grads, n_atoms, bwd_bytes))
 
     cpu = None
     if not args.no_cpu:
@@ -346,6 +405,7 @@ def main():
                    "batch": B, "atoms": n_atoms, "grid": [T, D, D, D]},
         "roofline": roofline,
         "kernels": kernels,
+        "parity": parity,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

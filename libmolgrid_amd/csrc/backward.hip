@@ -225,9 +225,9 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
         }
       }
     }
-    gx = wave_sum(gx) * gauss;
-    gy = wave_sum(gy) * gauss;
-    gz = wave_sum(gz) * gauss;
+    gx = (float)(wave_sum64(gx) * (double)gauss);
+    gy = (float)(wave_sum64(gy) * (double)gauss);
+    gz = (float)(wave_sum64(gz) * (double)gauss);
     if (lane == 0) {
       atom_gradients[3 * a] = gx;
       atom_gradients[3 * a + 1] = gy;

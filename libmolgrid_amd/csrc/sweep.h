@@ -18,22 +18,28 @@ constexpr int kDppRowBcast15 = 0x142;
 constexpr int kDppRowBcast31 = 0x143;
 
 template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add(float v) {
+__device__ __forceinline__ double dpp_add(double v) {
   // lanes outside ROW_MASK (or without a source lane) contribute 0
-  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
-  return v + __int_as_float(moved);
+  const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, ROW_MASK, 0xF, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, ROW_MASK, 0xF, false);
+  return v + __hiloint2double(hi, lo);
 }
 
-// Sum of v over the 64 lanes of the wave, returned to every lane.
-__device__ __forceinline__ float wave_sum(float v) {
+// Sum of v over the 64 lanes of the wave, returned to every lane.  The lanes' float partial sums
+// are added in double: the cross-lane step adds no rounding of its own (the reference's
+// sequential float loop, src/grid_maker.cu:898-919, carries more).
+__device__ __forceinline__ double wave_sum64(float value) {
+  double v = (double)value;
   v = dpp_add<kDppQuadPerm1032, 0xF>(v);
   v = dpp_add<kDppQuadPerm2301, 0xF>(v);
   v = dpp_add<kDppRowHalfMirror, 0xF>(v);
   v = dpp_add<kDppRowMirror, 0xF>(v);   // every lane of a 16-lane row holds the row total
   v = dpp_add<kDppRowBcast15, 0xA>(v);  // rows 1 and 3 add the total of rows 0 and 2
   v = dpp_add<kDppRowBcast31, 0xC>(v);  // rows 2 and 3 add the total of rows 0..1
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), 63),
+                          __builtin_amdgcn_readlane(__double2loint(v), 63));
 }
+__device__ __forceinline__ float wave_sum(float v) { return (float)wave_sum64(v); }
 
 // Sweep of an atom's voxel box [lo, lo+n) by one wave.  Each lane owns one (y, z) column of the
 // box (64 columns per pass) and marches along x, so everything that depends on y and z only --

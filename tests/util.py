@@ -37,3 +37,18 @@ def rot_matrix(q):
         [a * a + b * b - c * c - d * d, 2 * (b * c - a * d), 2 * (b * d + a * c)],
         [2 * (b * c + a * d), a * a - b * b + c * c - d * d, 2 * (c * d - a * b)],
         [2 * (b * d - a * c), 2 * (c * d + a * b), a * a - b * b - c * c + d * d]]) / n
+
+
+def parity_stats(got, ref, rtol=RTOL, atol=ATOL):
+    """Measured distance of `got` from `ref`: largest absolute error, largest relative error
+    (over |ref| > 1e-3), and how many values lie outside atol + rtol*|ref|."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    err = np.abs(got - ref)
+    big = np.abs(ref) > 1e-3
+    return {
+        "n": int(err.size),
+        "max_abs": float(err.max()) if err.size else 0.0,
+        "max_rel": float((err[big] / np.abs(ref[big])).max()) if big.any() else 0.0,
+        "outside": int((err > atol + rtol * np.abs(ref)).sum()),
+    }
