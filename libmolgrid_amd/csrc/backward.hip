@@ -135,7 +135,9 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
       const float inv_ar = 1.0f / ar;
       const float inv_ar2 = inv_ar * inv_ar;
       const float exp_k = inv_ar2 * kNeg2Log2e;
-      gauss = 4.0f * inv_ar2;
+      // an atom without extent (the padding rows of a padded batch) has no gradient, as in the
+      // reference, whose distance test fails for every voxel of such an atom
+      gauss = ar > 0.f ? 4.0f * inv_ar2 : 0.f;
       const float quad_a = -0.25f * g.D;
       const float quad_b = -0.25f * g.E * ar;
       const float core2 = g.grm * g.grm * ar * ar;
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
       reach_range(ox, ax, densityrad, inv_res, dim, lo0, ni);
       reach_range(oy, ay, densityrad, inv_res, dim, lo1, nj);
       reach_range(oz, az, densityrad, inv_res, dim, lo2, nk);
-      if (ni > 0 && nj > 0 && nk > 0) {
+      if (ni > 0 && nj > 0 && nk > 0 && ar > 0.f) {
         const float* chan = diff_b + (size_t)(int)tf * chan_stride;
         const int ncols = nj * nk;
         const float inv_nk = __builtin_amdgcn_rcpf((float)nk);
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
       bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
       bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
       const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
-      const bool any = ni > 0 && nj > 0 && nk > 0;
+      const bool any = ni > 0 && nj > 0 && nk > 0 && ar > 0.f;   // no extent: no gradient
       for (int cbase = 0; cbase < T; cbase += TG) {
         const int nchan = min(TG, T - cbase);
         float tg[TG];
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
         const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
         float tgt = 0.f, tx = 0.f, ty = 0.f, tz = 0.f;
-        if (ni > 0 && nj > 0 && nk > 0) {
+        if (ni > 0 && nj > 0 && nk > 0 && ar > 0.f) {
           const float* chan = diff_b + (size_t)t * chan_stride;
           sweep_channel(g, chan, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
                         [&](float dx, float dy, float dz, float dist2, float gv, bool live) {

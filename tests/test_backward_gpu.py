@@ -211,3 +211,25 @@ def test_argument_errors(mg):
     with pytest.raises(ValueError):
         mg.GridMaker(0.5, 7.5, False, True).backward((0, 0, 0), z(4, 3), z(4), z(4),
                                                      z(2, 16, 16, 16), z(4, 3))
+
+
+def test_padding_atoms_without_radius_get_zero_gradient(mg):
+    """The rows that pad a batch (radius 0, coordinates 0) sit exactly on a voxel centre when the
+    grid is centred at the origin with an odd number of points: their gradient is 0, as in the
+    reference (its distance test fails for every voxel of such an atom), not NaN."""
+    rng = np.random.default_rng(21)
+    coords, types, radii = synth.small_index_case(rng, 30, 3, 4.0, frac_ignored=0.0)
+    coords = np.concatenate([coords, np.zeros((4, 3), np.float32)])
+    types = np.concatenate([types, np.zeros(4, np.float32)])
+    radii = np.concatenate([radii, np.zeros(4, np.float32)])
+    gm = mg.GridMaker(0.5, 8.0)                 # 17 points a side: a voxel centre at the origin
+    og = oracle.GridMaker(0.5, 8.0)
+    diff = rng.standard_normal(gm.grid_dimensions(3)).astype(np.float32)
+    grads = torch.full((34, 3), 7.0, device="cuda")
+    gm.backward((0, 0, 0), dev(coords), dev(types), dev(radii), dev(diff), grads)
+    got = grads.cpu().numpy()
+    assert np.all(got[30:] == 0.0) and np.isfinite(got).all()
+    args = ((0, 0, 0), coords, types, radii, diff)
+    ref = og.backward(*args)
+    assert np.all(ref[30:] == 0.0)
+    check_grads(got, ref, og.backward(*args, f64=True), noise_bound(og, *args), "padded")
