@@ -1,6 +1,6 @@
 // GridMaker: atoms -> density grid (forward) and grid gradient -> atom / type gradients (backward).
 // Same constructor, accessors and forward/backward overload set as libmolgrid's GridMaker
-// (include/libmolgrid/grid_maker.h:34-445) for single precision grids.  Argument checks throw the
+// (include/libmolgrid/grid_maker.h:34-445); double precision grids are staged through float copies.  Argument checks throw the
 // reference's exception types (src/grid_maker.cpp:39-89, 442-451, 487-498); the numeric work is
 // one call into the C ABI per overload.  Overloads on host grids (isCUDA = false) stage their
 // arrays through device memory -- the kernels are the only implementation.
@@ -20,10 +20,12 @@ class GridMaker {
   mg_gridmaker p;           // resolution, dimension, radius multiples, A..E, dim, flags
   float grm_as_given = 1.0; // gaussian_radius_multiple as passed in (may be negative)
 
+  /// the second-order pass exists for single precision grids only, as in the reference
+  /// (src/grid_maker.cu:805: one instantiation, float)
   template <typename Dtype>
   static void require_float() {
     if (!std::is_same<Dtype, float>::value)
-      throw std::invalid_argument("double precision grids are not supported by the HIP gridding kernels");
+      throw std::invalid_argument("backward_gradients works on single precision grids");
   }
   void reinit(float res, float d) {
     abi_check(mg_gridmaker_init(&p, res, d, p.binary, p.radii_type_indexed, p.radius_scale, grm_as_given),
@@ -149,7 +151,6 @@ class GridMaker {
   template <typename Dtype, bool isCUDA>
   void forward(const std::vector<Example>& in, Grid<Dtype, 5, isCUDA>& out, float random_translation = 0.0,
                bool random_rotation = false) const {
-    require_float<Dtype>();
     if (in.size() != out.dimension(0))
       throw std::out_of_range("output grid dimension does not match size of example vector");
     const size_t B = in.size();
@@ -207,17 +208,20 @@ class GridMaker {
       abi_check(mg_transform_forward((int)B, doff.get(), longest, dq.get(), ident, dcen.get(), zero3, dsh.get(), zero3,
                                      1, dc.get(), dc.get(), nullptr),
                 "GridMaker::forward");
+    detail::AsFloat<Dtype, 5, isCUDA> f_out(out, false);
     if (isCUDA) {
       abi_check(mg_forward_index(&p, (int)B, doff.get(), longest, dcen.get(), zero3, dc.get(), dt.get(), dr.get(),
-                                 (int)out.dimension(1), reinterpret_cast<float*>(out.data()), nullptr),
+                                 (int)out.dimension(1), f_out.grid().data(), nullptr),
                 "GridMaker::forward");
+      f_out.commit();
       LMG_HIP_CHECK(hipDeviceSynchronize());  // the staged inputs are released on return
     } else {
       detail::DeviceStaging<float> dout(out.size());
       abi_check(mg_forward_index(&p, (int)B, doff.get(), longest, dcen.get(), zero3, dc.get(), dt.get(), dr.get(),
                                  (int)out.dimension(1), dout.get(), nullptr),
                 "GridMaker::forward");
-      dout.download(reinterpret_cast<float*>(out.data()));
+      dout.download(f_out.grid().data());
+      f_out.commit();
     }
   }
 
@@ -225,20 +229,21 @@ class GridMaker {
   template <typename Dtype>
   void forward(float3 grid_center, const Grid<float, 2, true>& coords, const Grid<float, 1, true>& type_index,
                const Grid<float, 1, true>& radii, Grid<Dtype, 4, true>& out) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, true> f_out(out, false);
     check_index_args(coords, type_index, radii, out);
     if (p.radii_type_indexed) throw std::invalid_argument("Type indexed radii not supported with index types.");
     const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
     abi_check(mg_forward_index(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
                                type_index.data(), radii.data(), (int)out.dimension(0),
-                               reinterpret_cast<float*>(out.data()), nullptr),
+                               f_out.grid().data(), nullptr),
               "GridMaker::forward");
+    f_out.commit();
   }
   /// index types, host arrays
   template <typename Dtype>
   void forward(float3 grid_center, const Grid<float, 2, false>& coords, const Grid<float, 1, false>& type_index,
                const Grid<float, 1, false>& radii, Grid<Dtype, 4, false>& out) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, false> f_out(out, false);
     check_index_args(coords, type_index, radii, out);
     if (p.radii_type_indexed) throw std::invalid_argument("Type indexed radii not supported with index types.");
     const size_t n = coords.dimension(0);
@@ -253,26 +258,28 @@ class GridMaker {
     Grid<float, 1, true> gt(dt.get(), n), gr(dr.get(), n);
     Grid<float, 4, true> go(dout.get(), out.dimension(0), out.dimension(1), out.dimension(2), out.dimension(3));
     forward(grid_center, gc, gt, gr, go);
-    dout.download(reinterpret_cast<float*>(out.data()));
+    dout.download(f_out.grid().data());
+    f_out.commit();
   }
 
   /// vector types, device arrays: one launch
   template <typename Dtype>
   void forward(float3 grid_center, const Grid<float, 2, true>& coords, const Grid<float, 2, true>& type_vector,
                const Grid<float, 1, true>& radii, Grid<Dtype, 4, true>& out) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, true> f_out(out, false);
     check_vector_args(coords, type_vector, radii, out);
     const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
     abi_check(mg_forward_vector(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
                                 type_vector.data(), radii.data(), (int)out.dimension(0),
-                                reinterpret_cast<float*>(out.data()), nullptr),
+                                f_out.grid().data(), nullptr),
               "GridMaker::forward");
+    f_out.commit();
   }
   /// vector types, host arrays
   template <typename Dtype>
   void forward(float3 grid_center, const Grid<float, 2, false>& coords, const Grid<float, 2, false>& type_vector,
                const Grid<float, 1, false>& radii, Grid<Dtype, 4, false>& out) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, false> f_out(out, false);
     check_vector_args(coords, type_vector, radii, out);
     const size_t n = coords.dimension(0), T = type_vector.dimension(1);
     detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_vector.data(), n * T), dr(radii.data(), radii.size());
@@ -281,7 +288,8 @@ class GridMaker {
     Grid<float, 1, true> gr(dr.get(), radii.size());
     Grid<float, 4, true> go(dout.get(), out.dimension(0), out.dimension(1), out.dimension(2), out.dimension(3));
     forward(grid_center, gc, gt, gr, go);
-    dout.download(reinterpret_cast<float*>(out.data()));
+    dout.download(f_out.grid().data());
+    f_out.commit();
   }
 
   /// padded batch: centers (B x 3), coords (B x N x 3), types (B x N) or (B x N x T), radii (B x N)
@@ -291,7 +299,6 @@ class GridMaker {
                const Grid<float, N, isCUDA>& types, const Grid<float, 2, isCUDA>& radii,
                Grid<Dtype, 5, isCUDA>& out) const {
     static_assert(N == 2 || N == 3, "Unsupported types dimension");
-    require_float<Dtype>();
     const size_t B = centers.dimension(0);
     if (coords.dimension(0) != B) throw std::invalid_argument("Mismatched batch sizes: " + itoa(coords.dimension(0)) + " vs " + itoa(B));
     if (types.dimension(0) != B) throw std::invalid_argument("Mismatched batch sizes: " + itoa(types.dimension(0)) + " vs " + itoa(B));
@@ -312,9 +319,11 @@ class GridMaker {
     }
     const int n = (int)coords.dimension(1);
     auto fn = N == 2 ? mg_forward_index : mg_forward_vector;
+    detail::AsFloat<Dtype, 5, isCUDA> f_out(out, false);
     abi_check(fn(&p, (int)B, nullptr, n, centers.data(), nullptr, coords.data(), types.data(), radii.data(),
-                 (int)out.dimension(1), reinterpret_cast<float*>(out.data()), nullptr),
+                 (int)out.dimension(1), f_out.grid().data(), nullptr),
               "GridMaker::forward");
+    f_out.commit();
   }
 
   // ---- backward --------------------------------------------------------------------------
@@ -351,21 +360,23 @@ class GridMaker {
   void backward(float3 grid_center, const Grid<float, 2, true>& coords, const Grid<float, 1, true>& type_index,
                 const Grid<float, 1, true>& radii, const Grid<Dtype, 4, true>& diff,
                 Grid<Dtype, 2, true>& atom_gradients) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, true> f_diff(diff, true);
+    detail::AsFloat<Dtype, 2, true> f_grad(atom_gradients, false);
     check_backward_index(coords, type_index, radii, diff, atom_gradients);
     const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
     abi_check(mg_backward_index(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
                                 type_index.data(), radii.data(), (int)diff.dimension(0),
-                                reinterpret_cast<const float*>(diff.data()),
-                                reinterpret_cast<float*>(atom_gradients.data()), nullptr),
+                                f_diff.grid().data(), f_grad.grid().data(), nullptr),
               "GridMaker::backward");
+    f_grad.commit();
   }
   /// index types, host arrays
   template <typename Dtype>
   void backward(float3 grid_center, const Grid<float, 2, false>& coords, const Grid<float, 1, false>& type_index,
                 const Grid<float, 1, false>& radii, const Grid<Dtype, 4, false>& diff,
                 Grid<Dtype, 2, false>& atom_gradients) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, false> f_diff(diff, true);
+    detail::AsFloat<Dtype, 2, false> f_grad(atom_gradients, false);
     check_backward_index(coords, type_index, radii, diff, atom_gradients);
     const size_t n = coords.dimension(0);
     for (size_t i = 0; i < n; ++i) {
@@ -374,12 +385,13 @@ class GridMaker {
         throw std::invalid_argument("Incorrect channel size for diff: " + itoa(which) + " vs " + itoa(diff.dimension(0)));
     }
     detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_index.data(), n), dr(radii.data(), n);
-    detail::DeviceStaging<float> dd(reinterpret_cast<const float*>(diff.data()), diff.size()), dg(n * 3);
+    detail::DeviceStaging<float> dd(f_diff.grid().data(), diff.size()), dg(n * 3);
     Grid<float, 2, true> gc(dc.get(), n, 3), gg(dg.get(), n, 3);
     Grid<float, 1, true> gt(dt.get(), n), gr(dr.get(), n);
     Grid<float, 4, true> gd(dd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
     backward(grid_center, gc, gt, gr, gd, gg);
-    dg.download(reinterpret_cast<float*>(atom_gradients.data()));
+    dg.download(f_grad.grid().data());
+    f_grad.commit();
   }
 
   /// vector types, device arrays
@@ -387,32 +399,36 @@ class GridMaker {
   void backward(float3 grid_center, const Grid<float, 2, true>& coords, const Grid<float, 2, true>& type_vectors,
                 const Grid<float, 1, true>& radii, const Grid<Dtype, 4, true>& diff,
                 Grid<Dtype, 2, true>& atom_gradients, Grid<Dtype, 2, true>& type_gradients) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, true> f_diff(diff, true);
+    detail::AsFloat<Dtype, 2, true> f_grad(atom_gradients, false), f_tgrad(type_gradients, false);
     check_backward_vector(coords, type_vectors, radii, diff, atom_gradients, type_gradients);
     const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
     abi_check(mg_backward_vector(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
                                  type_vectors.data(), radii.data(), (int)diff.dimension(0),
-                                 reinterpret_cast<const float*>(diff.data()),
-                                 reinterpret_cast<float*>(atom_gradients.data()),
-                                 reinterpret_cast<float*>(type_gradients.data()), nullptr),
+                                 f_diff.grid().data(), f_grad.grid().data(), f_tgrad.grid().data(), nullptr),
               "GridMaker::backward");
+    f_grad.commit();
+    f_tgrad.commit();
   }
   /// vector types, host arrays
   template <typename Dtype>
   void backward(float3 grid_center, const Grid<float, 2, false>& coords, const Grid<float, 2, false>& type_vectors,
                 const Grid<float, 1, false>& radii, const Grid<Dtype, 4, false>& diff,
                 Grid<Dtype, 2, false>& atom_gradients, Grid<Dtype, 2, false>& type_gradients) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, false> f_diff(diff, true);
+    detail::AsFloat<Dtype, 2, false> f_grad(atom_gradients, false), f_tgrad(type_gradients, false);
     check_backward_vector(coords, type_vectors, radii, diff, atom_gradients, type_gradients);
     const size_t n = coords.dimension(0), T = type_vectors.dimension(1);
     detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_vectors.data(), n * T), dr(radii.data(), radii.size());
-    detail::DeviceStaging<float> dd(reinterpret_cast<const float*>(diff.data()), diff.size()), dg(n * 3), dtg(n * T);
+    detail::DeviceStaging<float> dd(f_diff.grid().data(), diff.size()), dg(n * 3), dtg(n * T);
     Grid<float, 2, true> gc(dc.get(), n, 3), gt(dt.get(), n, T), gg(dg.get(), n, 3), gtg(dtg.get(), n, T);
     Grid<float, 1, true> gr(dr.get(), radii.size());
     Grid<float, 4, true> gd(dd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
     backward(grid_center, gc, gt, gr, gd, gg, gtg);
-    dg.download(reinterpret_cast<float*>(atom_gradients.data()));
-    dtg.download(reinterpret_cast<float*>(type_gradients.data()));
+    dg.download(f_grad.grid().data());
+    dtg.download(f_tgrad.grid().data());
+    f_grad.commit();
+    f_tgrad.commit();
   }
 
   // ---- relevance (include/libmolgrid/grid_maker.h:547-618 of the reference) ----------------
@@ -422,15 +438,15 @@ class GridMaker {
                           const Grid<float, 1, true>& type_index, const Grid<float, 1, true>& radii,
                           const Grid<Dtype, 4, true>& density, const Grid<Dtype, 4, true>& diff,
                           Grid<Dtype, 1, true>& relevance) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, true> f_dens(density, true), f_diff(diff, true);
+    detail::AsFloat<Dtype, 1, true> f_rel(relevance, false);
     check_relevance(coords, type_index, radii, density, diff, relevance);
     const float c[3] = {grid_center.x, grid_center.y, grid_center.z};
     abi_check(mg_backward_relevance(&p, 1, nullptr, (int)coords.dimension(0), nullptr, c, coords.data(),
                                     type_index.data(), radii.data(), (int)diff.dimension(0),
-                                    reinterpret_cast<const float*>(density.data()),
-                                    reinterpret_cast<const float*>(diff.data()),
-                                    reinterpret_cast<float*>(relevance.data()), nullptr),
+                                    f_dens.grid().data(), f_diff.grid().data(), f_rel.grid().data(), nullptr),
               "GridMaker::backward_relevance");
+    f_rel.commit();
   }
   /// index types, host arrays
   template <typename Dtype>
@@ -438,18 +454,20 @@ class GridMaker {
                           const Grid<float, 1, false>& type_index, const Grid<float, 1, false>& radii,
                           const Grid<Dtype, 4, false>& density, const Grid<Dtype, 4, false>& diff,
                           Grid<Dtype, 1, false>& relevance) const {
-    require_float<Dtype>();
+    detail::AsFloat<Dtype, 4, false> f_dens(density, true), f_diff(diff, true);
+    detail::AsFloat<Dtype, 1, false> f_rel(relevance, false);
     check_relevance(coords, type_index, radii, density, diff, relevance);
     const size_t n = coords.dimension(0);
     detail::DeviceStaging<float> dc(coords.data(), n * 3), dt(type_index.data(), n), dr(radii.data(), n);
-    detail::DeviceStaging<float> dd(reinterpret_cast<const float*>(density.data()), density.size());
-    detail::DeviceStaging<float> df(reinterpret_cast<const float*>(diff.data()), diff.size()), drel(n);
+    detail::DeviceStaging<float> dd(f_dens.grid().data(), density.size());
+    detail::DeviceStaging<float> df(f_diff.grid().data(), diff.size()), drel(n);
     Grid<float, 2, true> gc(dc.get(), n, 3);
     Grid<float, 1, true> gt(dt.get(), n), gr(dr.get(), n), grel(drel.get(), n);
     Grid<float, 4, true> gd(dd.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
     Grid<float, 4, true> gf(df.get(), diff.dimension(0), diff.dimension(1), diff.dimension(2), diff.dimension(3));
     backward_relevance(grid_center, gc, gt, gr, gd, gf, grel);
-    drel.download(reinterpret_cast<float*>(relevance.data()));
+    drel.download(f_rel.grid().data());
+    f_rel.commit();
   }
   /// coordinate set (host / device grids)
   template <typename Dtype>

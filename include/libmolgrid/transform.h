@@ -5,6 +5,7 @@
 #define LIBMOLGRID_TRANSFORM_H_
 
 #include <cmath>
+#include <vector>
 
 #include "libmolgrid/coordinateset.h"
 #include "libmolgrid/libmolgrid.h"
@@ -33,6 +34,64 @@ class DeviceStaging {
   void download(T* host) const {
     LMG_HIP_CHECK(hipDeviceSynchronize());
     raw_copy(host, false, ptr, true, count);
+  }
+};
+
+/// A float stand-in for a caller's grid.  For a float grid it is the grid itself.  For a double
+/// grid -- the reference instantiates its overloads for Grid<double, ...> as well and computes in
+/// float there too (src/grid_maker.cu:293-294, 445-446, 600; src/transform.cu:96) -- it is a float
+/// copy, on the device for a device grid and on the host for a host grid: filled from the grid
+/// when `load` is set, written back to it by commit().
+template <typename Dtype, int N, bool isCUDA>
+class AsFloat;
+
+template <int N, bool isCUDA>
+class AsFloat<float, N, isCUDA> {
+  Grid<float, N, isCUDA> g;
+
+ public:
+  AsFloat(const Grid<float, N, isCUDA>& src, bool) : g(src) {}
+  Grid<float, N, isCUDA>& grid() { return g; }
+  void commit() {}
+};
+
+template <int N>
+class AsFloat<double, N, true> {
+  DeviceStaging<float> buf;
+  double* orig;
+  size_t count;
+  Grid<float, N, true> g;
+
+ public:
+  AsFloat(const Grid<double, N, true>& src, bool load)
+      : buf(src.size()), orig(const_cast<double*>(src.data())), count(src.size()) {
+    size_t d[N];
+    for (int i = 0; i < N; ++i) d[i] = src.dimension(i);
+    g = Grid<float, N, true>(buf.get(), d);
+    if (load) abi_check(mg_narrow(orig, buf.get(), count, nullptr), "double grid");
+  }
+  Grid<float, N, true>& grid() { return g; }
+  void commit() { abi_check(mg_widen(buf.get(), orig, count, nullptr), "double grid"); }
+};
+
+template <int N>
+class AsFloat<double, N, false> {
+  std::vector<float> buf;
+  double* orig;
+  Grid<float, N, false> g;
+
+ public:
+  AsFloat(const Grid<double, N, false>& src, bool load)
+      : buf(src.size()), orig(const_cast<double*>(src.data())) {
+    size_t d[N];
+    for (int i = 0; i < N; ++i) d[i] = src.dimension(i);
+    g = Grid<float, N, false>(buf.data(), d);
+    if (load)
+      for (size_t i = 0; i < buf.size(); ++i) buf[i] = (float)orig[i];
+  }
+  Grid<float, N, false>& grid() { return g; }
+  void commit() {
+    for (size_t i = 0; i < buf.size(); ++i) orig[i] = (double)buf[i];
   }
 };
 }  // namespace detail
@@ -66,18 +125,18 @@ class Transform {
   template <typename Dtype, bool isCUDA>
   void apply(bool inverse, const Grid<Dtype, 2, isCUDA>& in, Grid<Dtype, 2, isCUDA>& out,
              bool dotranslate) const {
-    static_assert(std::is_same<Dtype, float>::value,
-                  "the HIP gridding kernels work on single precision coordinates");
     checkGrids(in, out);
     const size_t n = in.dimension(0);
     if (n == 0) return;
+    detail::AsFloat<Dtype, 2, isCUDA> f_in(in, true), f_out(out, false);
     if (isCUDA) {
-      launch(inverse, in.data(), out.data(), n, dotranslate);
+      launch(inverse, f_in.grid().data(), f_out.grid().data(), n, dotranslate);
     } else {
-      detail::DeviceStaging<float> buf(in.data(), n * 3);
+      detail::DeviceStaging<float> buf(f_in.grid().data(), n * 3);
       launch(inverse, buf.get(), buf.get(), n, dotranslate);
-      buf.download(out.data());
+      buf.download(f_out.grid().data());
     }
+    f_out.commit();
   }
 
  public:

@@ -216,6 +216,16 @@ int mg_interpolate(float in_resolution, float in_dimension, float out_resolution
                    const float* out_centers, const float out_center_host[3], float* out,
                    void* stream);
 
+/* Double precision arrays at the boundary.  The reference instantiates its GPU
+ * overloads for Grid<double, N, true> outputs, gradients and coordinates too
+ * (src/grid_maker.cu:293-294, 445-446, 460-466, 600; src/transform.cu:96;
+ * torch.cuda.DoubleTensor in python/bindings_grids.cpp:108-116) and computes in
+ * float there as here.  The kernels of this library read and write float; the
+ * host layers stage a double array through a float copy with these two:
+ *   mg_narrow: dst[i] = (float)src[i]     mg_widen: dst[i] = (double)src[i] */
+int mg_narrow(const double* src, float* dst, size_t n, void* stream);
+int mg_widen(const float* src, double* dst, size_t n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libmolgrid_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
-SOURCES = ["capi.hip", "transform.hip", "forward_sorted.hip", "forward_vector.hip", "forward_vector_mfma.hip",
+SOURCES = ["capi.hip", "transform.hip", "convert.hip", "forward_sorted.hip", "forward_vector.hip", "forward_vector_mfma.hip",
            "backward.hip", "second_order.hip", "interpolate.hip"]
 
 # Packed FP32 instructions are kept out of the generated code.

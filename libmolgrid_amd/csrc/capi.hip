@@ -418,6 +418,18 @@ int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom
                                             (hipStream_t)stream));
 }
 
+int mg_widen(const float* src, double* dst, size_t n, void* stream) {
+  if (n == 0) return MG_OK;
+  if (src == nullptr || dst == nullptr) return MG_ERR_NULL_POINTER;
+  return from_hip(launch_widen(src, dst, n, (hipStream_t)stream));
+}
+
+int mg_narrow(const double* src, float* dst, size_t n, void* stream) {
+  if (n == 0) return MG_OK;
+  if (src == nullptr || dst == nullptr) return MG_ERR_NULL_POINTER;
+  return from_hip(launch_narrow(src, dst, n, (hipStream_t)stream));
+}
+
 int mg_interpolate(float in_resolution, float in_dimension, float out_resolution,
                    float out_dimension, int nbatch, int channels, const float* in_centers,
                    const float in_center_host[3], const float* in, const float* quats,

@@ -79,6 +79,10 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
                               const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,
                               hipStream_t stream);
 
+// float <-> double copies (convert.hip)
+hipError_t launch_widen(const float* src, double* dst, size_t n, hipStream_t stream);
+hipError_t launch_narrow(const double* src, float* dst, size_t n, hipStream_t stream);
+
 }  // namespace mg
 
 #endif

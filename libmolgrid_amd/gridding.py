@@ -189,36 +189,47 @@ class _Arg(object):
     """A user array made visible to the device.
 
     ROCm tensors are used in place after the checks of
-    python/bindings_grids.cpp:91-137 (float32, contiguous, on the current
-    device).  Host arrays are copied to the device when the pointer is first
-    asked for (after all shape checks have passed) and, for outputs, back.
+    python/bindings_grids.cpp:91-137 (contiguous, on the current device).  Host
+    arrays are copied to the device when the pointer is first asked for (after
+    all shape checks have passed) and, for outputs, back.
+
+    The kernels read and write float32.  Where the reference has a
+    ``Grid<double, ...>`` overload (``wide=True``: output grids, upstream
+    gradients and gradients, transformed coordinates;
+    python/bindings_grids.cpp:108-116) a float64 array is staged through a
+    float32 copy on the device: narrowed before the call, widened after it.
     """
 
-    def __init__(self, x, name, ndim, out=False):
+    def __init__(self, x, name, ndim, out=False, wide=False):
         x = _unwrap(x)
         self.name = name
         self.out = out
         self.host = None
         self.t = None
+        self.wide_dev = None        # the caller's float64 device tensor, if that is what came
         if isinstance(x, torch.Tensor) and x.is_cuda:
-            if x.dtype != torch.float32:
+            if x.dtype != torch.float32 and not (wide and x.dtype == torch.float64):
                 raise ValueError("%s: only float32 device tensors are supported" % name)
             if not x.is_contiguous():
                 raise ValueError("%s: tensor is not contiguous" % name)
             if x.device.index != torch.cuda.current_device():
                 raise ValueError("%s: tensor is on device %d but the current device is %d"
                                  % (name, x.device.index, torch.cuda.current_device()))
-            self.t = x
+            if x.dtype == torch.float64:
+                self.wide_dev = x
+            else:
+                self.t = x
             self.shape = tuple(x.shape)
         else:
             if isinstance(x, torch.Tensor):
-                if x.dtype != torch.float32:
+                if x.dtype != torch.float32 and not (wide and x.dtype == torch.float64):
                     raise ValueError("%s: only float32 tensors are supported" % name)
                 if not x.is_contiguous():
                     raise ValueError("%s: tensor is not contiguous" % name)
                 self.host = x.detach()
             elif out:
-                if not (isinstance(x, np.ndarray) and x.dtype == np.float32
+                ok = (np.float32, np.float64) if wide else (np.float32,)
+                if not (isinstance(x, np.ndarray) and x.dtype in ok
                         and x.flags.c_contiguous and x.flags.writeable):
                     raise ValueError("%s: output must be a writable C-contiguous float32 "
                                      "array" % name)
@@ -232,13 +243,26 @@ class _Arg(object):
     @property
     def ptr(self):
         if self.t is None:
-            self.t = (torch.empty(self.shape, dtype=torch.float32, device=_device()) if self.out
-                      else self.host.to(_device()))
+            if self.out:
+                self.t = torch.empty(self.shape, dtype=torch.float32, device=_device())
+            elif self.wide_dev is not None:
+                self.t = torch.empty(self.shape, dtype=torch.float32, device=_device())
+                if self.t.numel():
+                    _capi.check(_lib.mg_narrow(self.wide_dev.data_ptr(), self.t.data_ptr(),
+                                               self.t.numel(), _stream()), self.name)
+            else:
+                self.t = self.host.to(device=_device(), dtype=torch.float32)
         return self.t.data_ptr() if self.t.numel() else None
 
     def finish(self):
-        if self.out and self.host is not None and self.t is not None:
-            self.host.copy_(self.t)
+        if not self.out or self.t is None:
+            return
+        if self.wide_dev is not None:
+            if self.t.numel():
+                _capi.check(_lib.mg_widen(self.t.data_ptr(), self.wide_dev.data_ptr(),
+                                          self.t.numel(), _stream()), self.name)
+        elif self.host is not None:
+            self.host.copy_(self.t)          # widens on the way when the host array is float64
 
 
 def _same_memory(a, b):
@@ -391,8 +415,8 @@ class Transform(object):
                 raise ValueError("Incompatible coordinateset sizes")
             src, dst = src.coords, dst.coords
         same = dst is src
-        a_in = _Arg(src, "in", 2)
-        a_out = a_in if same and not _is_host(src) else _Arg(dst, "out", 2, out=True)
+        a_in = _Arg(src, "in", 2, wide=True)
+        a_out = a_in if same and a_in.t is not None else _Arg(dst, "out", 2, out=True, wide=True)
         # transform.h:131-146 (checkGrids)
         if a_in.shape[0] != a_out.shape[0]:
             raise ValueError("Different dimensions and input and output coordinates grids.")
@@ -427,8 +451,8 @@ def transform_batch(offsets, quats, centers, translations, src, dst, dotranslate
     """
     off, nbatch, largest, total = _offsets_arg(offsets)
     q, c, t = _small_device(quats, 4), _small_device(centers, 3), _small_device(translations, 3)
-    a_in = _Arg(src, "in", 2)
-    a_out = a_in if dst is src and not _is_host(src) else _Arg(dst, "out", 2, out=True)
+    a_in = _Arg(src, "in", 2, wide=True)
+    a_out = a_in if dst is src and a_in.t is not None else _Arg(dst, "out", 2, out=True, wide=True)
     if a_in.shape != a_out.shape or a_in.shape[1] != 3 or a_in.shape[0] < total:
         raise ValueError("coordinate arrays must both be (n, 3) with n >= offsets[-1]")
     for name, v in (("quats", q), ("centers", c), ("translations", t)):
@@ -1089,7 +1113,7 @@ class GridMaker(object):
         tdim = len(tuple(types.shape))
         a_types = _Arg(types, "types", tdim)
         a_radii = _Arg(radii, "radii", 1)
-        a_out = _Arg(grid, "grid", 4, out=True)
+        a_out = _Arg(grid, "grid", 4, out=True, wide=True)
         n = a_coords.shape[0]
         if tdim == 1:
             self._check_index_args(n, a_types, a_radii, a_out.shape)
@@ -1175,7 +1199,7 @@ class GridMaker(object):
             raise ValueError("Unsupported types dimension")
         a_types = _Arg(types, "types", tdim)
         a_radii = _Arg(radii, "radii", 2)
-        a_out = _Arg(grid, "grid", 5, out=True)
+        a_out = _Arg(grid, "grid", 5, out=True, wide=True)
         B = a_centers.shape[0]
         for a in (a_coords, a_types, a_radii, a_out):
             if a.shape[0] != B:
@@ -1209,7 +1233,7 @@ class GridMaker(object):
         a_types = _Arg(types, "types", tdim)
         rti = bool(self._p.radii_type_indexed)
         a_radii = _Arg(radii, "radii", 2 if rti else 1)
-        a_out = _Arg(grid, "grid", 5, out=True)
+        a_out = _Arg(grid, "grid", 5, out=True, wide=True)
         if cen.shape[0] != B or a_out.shape[0] != B:
             raise ValueError("Mismatched batch sizes: %d vs %d" % (a_out.shape[0], B))
         if a_coords.shape[0] < total or a_types.shape[0] < total:
@@ -1263,8 +1287,8 @@ class GridMaker(object):
         tdim = len(tuple(types.shape))
         a_types = _Arg(types, "types", tdim)
         a_radii = _Arg(radii, "radii", 1)
-        a_diff = _Arg(diff, "diff", 4)
-        a_ag = _Arg(agrad, "atom_gradients", 2, out=True)
+        a_diff = _Arg(diff, "diff", 4, wide=True)
+        a_ag = _Arg(agrad, "atom_gradients", 2, out=True, wide=True)
         n = a_coords.shape[0]
         dim = int(self._p.dim)
         if tdim == 1:
@@ -1298,7 +1322,7 @@ class GridMaker(object):
             return
         if len(args) != 7:
             raise TypeError("vector types need a type_gradients argument")
-        a_tg = _Arg(args[6], "type_gradients", 2, out=True)
+        a_tg = _Arg(args[6], "type_gradients", 2, out=True, wide=True)
         T = a_types.shape[1]
         # src/grid_maker.cpp:487-498
         if n != a_types.shape[0]:
@@ -1348,9 +1372,9 @@ class GridMaker(object):
         a_coords = _Arg(coords, "coords", 2)
         a_types = _Arg(types, "type_index", 1)
         a_radii = _Arg(radii, "radii", 1)
-        a_dens = _Arg(density, "density", 4)
-        a_diff = _Arg(diff, "diff", 4)
-        a_rel = _Arg(relevance, "relevance", 1, out=True)
+        a_dens = _Arg(density, "density", 4, wide=True)
+        a_diff = _Arg(diff, "diff", 4, wide=True)
+        a_rel = _Arg(relevance, "relevance", 1, out=True, wide=True)
         n = a_coords.shape[0]
         # src/grid_maker.cu:975-978
         if n != a_types.shape[0]:
@@ -1392,7 +1416,7 @@ class GridMaker(object):
         a_coords = _Arg(coords, "coords", 2)
         a_types = _Arg(types, "type_vectors", 2)
         a_radii = _Arg(radii, "radii", 1)
-        a_diff = _Arg(diff, "diff", 4)
+        a_diff = _Arg(diff, "diff", 4, wide=True)
         a_ag = _Arg(agrad, "atom_gradients", 2)
         a_tg = _Arg(tgrad, "type_gradients", 2)
         a_dd = _Arg(diffdiff, "diffdiff", 4, out=True)
@@ -1444,8 +1468,8 @@ class GridMaker(object):
             raise ValueError("Unsupported types dimension")
         a_types = _Arg(types, "types", tdim)
         a_radii = _Arg(radii, "radii", 2)
-        a_diff = _Arg(diff, "diff", 5)
-        a_ag = _Arg(agrad, "atom_gradients", 3, out=True)
+        a_diff = _Arg(diff, "diff", 5, wide=True)
+        a_ag = _Arg(agrad, "atom_gradients", 3, out=True, wide=True)
         B, n = a_coords.shape[0], a_coords.shape[1]
         for a in (a_types, a_radii, a_diff, a_ag):
             if a.shape[0] != B:
@@ -1479,7 +1503,7 @@ class GridMaker(object):
             return
         if tgrad is None:
             raise TypeError("vector types need a type_gradients argument")
-        a_tg = _Arg(tgrad, "type_gradients", 3, out=True)
+        a_tg = _Arg(tgrad, "type_gradients", 3, out=True, wide=True)
         if a_types.shape[2] != T:
             raise ValueError("Channels in diff doesn't equal number of types")
         if a_tg.shape != a_types.shape:
@@ -1506,8 +1530,8 @@ class GridMaker(object):
         a_types = _Arg(types, "types", tdim)
         rti = bool(self._p.radii_type_indexed)
         a_radii = _Arg(radii, "radii", 2 if rti else 1)
-        a_diff = _Arg(diff, "diff", 5)
-        a_ag = _Arg(atom_gradients, "atom_gradients", 2, out=True)
+        a_diff = _Arg(diff, "diff", 5, wide=True)
+        a_ag = _Arg(atom_gradients, "atom_gradients", 2, out=True, wide=True)
         if cen.shape[0] != B or a_diff.shape[0] != B:
             raise ValueError("Mismatched batch sizes: %d vs %d" % (a_diff.shape[0], B))
         if a_ag.shape != a_coords.shape or a_coords.shape[1] != 3:
@@ -1531,7 +1555,7 @@ class GridMaker(object):
             return
         if type_gradients is None:
             raise TypeError("vector types need a type_gradients argument")
-        a_tg = _Arg(type_gradients, "type_gradients", 2, out=True)
+        a_tg = _Arg(type_gradients, "type_gradients", 2, out=True, wide=True)
         if a_types.shape[1] != T or a_tg.shape != a_types.shape:
             raise ValueError("Type gradient dimension has wrong number of types")
         if rti and a_radii.shape != (B, T):

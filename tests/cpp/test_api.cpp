@@ -229,6 +229,54 @@ static void gpu_tests() {
     CHECK(throws<std::invalid_argument>([&] { gb.backward_gradients(make_float3(0, 0, 0), cs, d4.gpu(), ag.gpu(), tg.gpu(), dd4.gpu(), add.gpu(), tdd.gpu()); }));
   }
 
+  // double precision grids (the reference's Grid<double, ...> overloads): the float result, widened
+  {
+    MGrid4d wide(3, 25, 25, 25), wide_host(3, 25, 25, 25);
+    MGrid4f narrow(3, 25, 25, 25);
+    CoordinateSet both = ex.merge_coordinates();
+    g1.forward(make_float3(0, 0, 0), both, narrow.gpu());
+    g1.forward(make_float3(0, 0, 0), both, wide.gpu());
+    g1.forward(make_float3(0, 0, 0), both, wide_host.cpu());
+    narrow.tocpu();
+    wide.tocpu();
+    bool same = true;
+    for (size_t i = 0; i < narrow.size(); ++i)
+      same = same && wide.cpu().data()[i] == (double)narrow.cpu().data()[i] &&
+             wide_host.cpu().data()[i] == (double)narrow.cpu().data()[i];
+    CHECK(same);
+    // backward: double upstream gradient and double atom gradients
+    MGrid4d dwide(3, 25, 25, 25);
+    MGrid4f dnarrow(3, 25, 25, 25);
+    for (size_t i = 0; i < dwide.size(); ++i) {
+      const float v = std::sin(0.37f * (float)i);
+      dnarrow.cpu().data()[i] = v;
+      dwide.cpu().data()[i] = v;
+    }
+    MGrid2d gwide(both.size(), 3), gwide_host(both.size(), 3);
+    MGrid2f gnarrow(both.size(), 3);
+    g1.backward(make_float3(0, 0, 0), both, dnarrow.gpu(), gnarrow.gpu());
+    g1.backward(make_float3(0, 0, 0), both, dwide.gpu(), gwide.gpu());
+    g1.backward(make_float3(0, 0, 0), both, dwide.cpu(), gwide_host.cpu());
+    gnarrow.tocpu();
+    gwide.tocpu();
+    same = true;
+    for (size_t i = 0; i < gnarrow.size(); ++i)
+      same = same && gwide.cpu().data()[i] == (double)gnarrow.cpu().data()[i] &&
+             gwide_host.cpu().data()[i] == (double)gnarrow.cpu().data()[i];
+    CHECK(same);
+    CHECK(gnarrow.cpu().data()[0] != 0.0f);
+    // Transform on double coordinates
+    MGrid2d cw(2, 3);
+    MGrid2f cn(2, 3);
+    for (int i = 0; i < 6; ++i) { cw.cpu().data()[i] = 0.5 * i - 1; cn.cpu().data()[i] = 0.5f * i - 1; }
+    Transform tq(Quaternion(std::sqrt(0.5f), 0, 0, std::sqrt(0.5f)), make_float3(0, 1, 0), make_float3(1, 2, 3));
+    tq.forward(cn.gpu(), cn.gpu());
+    tq.forward(cw.gpu(), cw.gpu());
+    cn.tocpu();
+    cw.tocpu();
+    for (int i = 0; i < 6; ++i) CHECK(cw.cpu().data()[i] == (double)cn.cpu().data()[i]);
+  }
+
   // batch of examples: one packed upload, two launches; equals the per-example calls bit for bit
   Example ex2;
   ex2.sets.push_back(CoordinateSet(p1, std::vector<int>{1}, std::vector<float>{2.0f}, 2));
