@@ -264,7 +264,13 @@ def main():
         mg.transform_batch(offsets, quats, centers, trans, grads, grads, dotranslate=False,
                            inverse=True)
 
+    def k_backward_unrotated():
+        gm.backward_batch(offsets, centers, moved, types, radii, diff, grads,
+                          unrotate=(quats, centers))
+
     def step():
+        # (k_backward_unrotated does the last two in one launch, bit for bit; it measures the
+        # same, see kernels.backward.unrotated_ms)
         k_transform()
         k_forward()
         k_backward()
@@ -305,6 +311,7 @@ def main():
     ms_bwd = event_ms(k_backward, it)
     ms_tr = event_ms(k_transform, it)
     in_step = step_breakdown([k_transform, k_forward, k_backward, k_unrotate], it)
+    ms_bwd_unrot = event_ms(k_backward_unrotated, it)
 
     grid_bytes = B * T * D ** 3 * 4
     fwd_bytes = grid_bytes + n_atoms * 20          # grid written once + coords/type/radius read
@@ -336,6 +343,7 @@ def main():
         "forward": {"ms": round(ms_fwd, 4), "in_step_ms": round(in_step[1], 4), "grids_per_s": round(B / (ms_fwd * 1e-3), 1),
                     "GBps": round(fwd_gbs, 1), "hbm_frac": round(fwd_gbs / HBM_PEAK_GBS, 4)},
         "backward": {"ms": round(ms_bwd, 4), "in_step_ms": round(in_step[2], 4),
+                     "unrotated_ms": round(ms_bwd_unrot, 4),
                      "atom_grads_per_s": round(n_atoms / (ms_bwd * 1e-3), 1),
                      "GBps": round(bwd_gbs, 1), "hbm_frac": round(bwd_gbs / HBM_PEAK_GBS, 4)},
         "transform": {"ms": round(ms_tr, 4), "in_step_ms": round(in_step[0], 4),

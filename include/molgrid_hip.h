@@ -166,6 +166,19 @@ int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
                       const float* type_index, const float* radii, int ntypes,
                       const float* diff, float* atom_gradients, void* stream);
 
+/* GridMaker::backward for index types followed by Transform::backward(gradients,
+ * dotranslate = false) per example -- the two calls of the reference's training
+ * loop (python/torch_bindings.py:124-136; src/grid_maker.cu:576-595,
+ * src/transform.cu:79-93) in one launch; the gradients are those the two calls
+ * give, bit for bit. */
+int mg_backward_index_unrotated(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                                int atoms_per_example, const float* grid_centers,
+                                const float grid_center_host[3], const float* coords,
+                                const float* type_index, const float* radii, int ntypes,
+                                const float* diff, const float* quats, const float quat_host[4],
+                                const float* rot_centers, const float rot_center_host[3],
+                                float* atom_gradients, void* stream);
+
 /* GridMaker::backward, vector types; replaces set_atom_type_gradients and its
  * launcher (src/grid_maker.cu:513-571, 604-642), values of
  * src/grid_maker.cpp:477-519.  type_gradients [n, ntypes] is overwritten. */

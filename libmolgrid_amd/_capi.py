@@ -20,6 +20,7 @@ EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
     "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_vector", "mg_backward_index",
+    "mg_backward_index_unrotated",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate",
     "mg_narrow", "mg_widen",
 )
@@ -72,6 +73,8 @@ def _load():
     lib.mg_forward_index_workspace_size.restype = ctypes.c_size_t
     lib.mg_forward_vector.argtypes = fwd
     lib.mg_backward_index.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp, _vp]
+    lib.mg_backward_index_unrotated.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp,
+                                                _vp, _f4, _vp, _f3, _vp, _vp]
     lib.mg_backward_vector.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,
                                        _vp, _vp]
     lib.mg_backward_relevance.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp,

@@ -91,10 +91,16 @@ __device__ __forceinline__ void reach_range(float origin, float coord, float rea
 // the offset in x of plane i is computed by lane i beforehand and read back as a scalar.  Per
 // voxel the lane adds scale*dx to its x partial and scale to a running sum: dy and dz are fixed
 // along the march, so the y and z partials are that sum times dy and dz.
+//
+// UNROTATE: the gradient is stored after Transform::backward(..., dotranslate = false) with the
+// example's quaternion and rotation centre, with the arithmetic of that call (transform.hip), so
+// that the result is the one the two calls give, bit for bit, with one launch less.
+template <bool UNROTATE>
 __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_index, const float* __restrict__ radii,
-    const float* __restrict__ diff, float* __restrict__ atom_gradients) {
+    const float* __restrict__ diff, float* __restrict__ atom_gradients, Vec4Arg quats,
+    Vec3Arg rot_centers) {
   // column list of each wave: (j << 16 | k) offsets inside the atom's box; a chunk of candidates
   // adds at most kWave entries to fewer than kWave pending ones
   __shared__ int s_cols[kBwdWaves][2 * kWave];
@@ -114,6 +120,18 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
   const float inv_res = 1.0f / g.resolution;
   volatile int* cols = s_cols[wave];
   constexpr int kPlanes = 16;   // planes of a column in flight together
+
+  // the inverse rotation of this example, once per wave
+  float4 un_q = make_float4(1.f, 0.f, 0.f, 0.f), un_qinv = un_q;
+  float3 un_c = make_float3(0.f, 0.f, 0.f), un_shift = un_c;
+  if (UNROTATE) {
+#pragma clang fp contract(off)
+    un_q = quat_inverse(load4(quats, b));
+    un_qinv = quat_inverse(un_q);
+    un_c = load3(rot_centers, b);
+    const float zero = 0.f;
+    un_shift = make_float3(-zero - un_c.x, -zero - un_c.y, -zero - un_c.z);
+  }
 
   for (int a = begin + blockIdx.x * kBwdWaves + wave; a < end; a += gridDim.x * kBwdWaves) {
     float gx = 0.f, gy = 0.f, gz = 0.f, gauss = 0.f;
@@ -230,6 +248,14 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
     gx = (float)(wave_sum64(gx) * (double)gauss);
     gy = (float)(wave_sum64(gy) * (double)gauss);
     gz = (float)(wave_sum64(gz) * (double)gauss);
+    if (UNROTATE) {
+      // src/transform.cpp:85-108 with dotranslate = false: rotate (g - c) by the inverse, add c
+#pragma clang fp contract(off)
+      const float3 r = quat_rotate(un_q, un_qinv, gx + un_shift.x, gy + un_shift.y, gz + un_shift.z);
+      gx = r.x + un_c.x;
+      gy = r.y + un_c.y;
+      gz = r.z + un_c.z;
+    }
     if (lane == 0) {
       atom_gradients[3 * a] = gx;
       atom_gradients[3 * a + 1] = gy;
@@ -406,8 +432,22 @@ hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nb
                                  const float* type_index, const float* radii, const float* diff,
                                  float* atom_gradients, hipStream_t stream) {
   dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
-  hipLaunchKernelGGL(backward_index_kernel, grid, block, 0, stream, g, batch, centers, coords,
-                     type_index, radii, diff, atom_gradients);
+  const Vec4Arg no_quats{nullptr, {1.f, 0.f, 0.f, 0.f}};
+  const Vec3Arg no_centers{nullptr, {0.f, 0.f, 0.f}};
+  hipLaunchKernelGGL(backward_index_kernel<false>, grid, block, 0, stream, g, batch, centers,
+                     coords, type_index, radii, diff, atom_gradients, no_quats, no_centers);
+  return hipGetLastError();
+}
+
+hipError_t launch_backward_index_unrotated(const GridArg& g, const BatchArg& batch, int nbatch,
+                                           int launch_atoms, const Vec3Arg& centers,
+                                           const float* coords, const float* type_index,
+                                           const float* radii, const float* diff,
+                                           const Vec4Arg& quats, const Vec3Arg& rot_centers,
+                                           float* atom_gradients, hipStream_t stream) {
+  dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
+  hipLaunchKernelGGL(backward_index_kernel<true>, grid, block, 0, stream, g, batch, centers,
+                     coords, type_index, radii, diff, atom_gradients, quats, rot_centers);
   return hipGetLastError();
 }
 

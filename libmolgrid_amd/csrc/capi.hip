@@ -351,6 +351,27 @@ int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
                                         (hipStream_t)stream));
 }
 
+int mg_backward_index_unrotated(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                                int atoms_per_example, const float* grid_centers,
+                                const float grid_center_host[3], const float* coords,
+                                const float* type_index, const float* radii, int ntypes,
+                                const float* diff, const float* quats, const float quat_host[4],
+                                const float* rot_centers, const float rot_center_host[3],
+                                float* atom_gradients, void* stream) {
+  int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (coords == nullptr || type_index == nullptr || radii == nullptr || diff == nullptr ||
+      atom_gradients == nullptr)
+    return MG_ERR_NULL_POINTER;
+  BatchArg batch{atom_offsets, atoms_per_example};
+  return from_hip(launch_backward_index_unrotated(
+      grid_arg(g, ntypes), batch, nbatch, atoms_per_example, vec3(grid_centers, grid_center_host),
+      coords, type_index, radii, diff, vec4(quats, quat_host), vec3(rot_centers, rot_center_host),
+      atom_gradients, (hipStream_t)stream));
+}
+
 int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                        int atoms_per_example, const float* grid_centers,
                        const float grid_center_host[3], const float* coords,

@@ -54,6 +54,14 @@ hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nb
                                  const float* type_index, const float* radii, const float* diff,
                                  float* atom_gradients, hipStream_t stream);
 
+// the same, followed by Transform::backward(gradients, dotranslate = false) per example
+hipError_t launch_backward_index_unrotated(const GridArg& g, const BatchArg& batch, int nbatch,
+                                           int launch_atoms, const Vec3Arg& centers,
+                                           const float* coords, const float* type_index,
+                                           const float* radii, const float* diff,
+                                           const Vec4Arg& quats, const Vec3Arg& rot_centers,
+                                           float* atom_gradients, hipStream_t stream);
+
 hipError_t launch_backward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
                                   int launch_atoms, const Vec3Arg& centers, const float* coords,
                                   const float* type_vector, const float* radii, const float* diff,

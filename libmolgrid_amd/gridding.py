@@ -1520,9 +1520,10 @@ class GridMaker(object):
 
     @_accepts_grids
     def backward_batch(self, offsets, centers, coords, types, radii, diff, atom_gradients,
-                       type_gradients=None):
+                       type_gradients=None, unrotate=None):
         """Ragged batch in one launch; diff is (B,T,D,D,D); gradients are packed like the
-        atom arrays."""
+        atom arrays.  ``unrotate=(quats, rotation_centers)`` (index types) also applies
+        ``Transform.backward(gradients, dotranslate=False)`` per example in the same launch."""
         off, B, largest, total = _offsets_arg(offsets)
         cen = _small_device(centers, 3)
         a_coords = _Arg(coords, "coords", 2)
@@ -1547,12 +1548,24 @@ class GridMaker(object):
         if tdim == 1:
             if rti:
                 raise ValueError("Type indexed radii not supported with index types.")
-            code = _lib.mg_backward_index(self._p, B, _ptr(off), largest, _ptr(cen),
-                                          _capi.f3(_Z3), a_coords.ptr, a_types.ptr, a_radii.ptr,
-                                          T, a_diff.ptr, a_ag.ptr, _stream())
+            if unrotate is not None:
+                q, rc = _small_device(unrotate[0], 4), _small_device(unrotate[1], 3)
+                if q.shape[0] != B or rc.shape[0] != B:
+                    raise ValueError("Mismatched batch sizes: the quaternions and rotation "
+                                     "centres need %d rows" % B)
+                code = _lib.mg_backward_index_unrotated(
+                    self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3), a_coords.ptr,
+                    a_types.ptr, a_radii.ptr, T, a_diff.ptr, _ptr(q), _capi.f4(_IDQ), _ptr(rc),
+                    _capi.f3(_Z3), a_ag.ptr, _stream())
+            else:
+                code = _lib.mg_backward_index(self._p, B, _ptr(off), largest, _ptr(cen),
+                                              _capi.f3(_Z3), a_coords.ptr, a_types.ptr,
+                                              a_radii.ptr, T, a_diff.ptr, a_ag.ptr, _stream())
             _capi.check(code, "GridMaker.backward_batch")
             a_ag.finish()
             return
+        if unrotate is not None:
+            raise ValueError("unrotate is for index types")
         if type_gradients is None:
             raise TypeError("vector types need a type_gradients argument")
         a_tg = _Arg(type_gradients, "type_gradients", 2, out=True, wide=True)

@@ -104,6 +104,15 @@ def test_backward_full_batch(mg, workload):
     assert gpu64["max_abs"] <= cpu64["max_abs"]
     excess = np.maximum(np.abs(got - ref64) - (1e-6 + 1e-5 * np.abs(ref64)), 0) / (EPS * mag)
     assert float(excess.max()) <= 16.0          # measured: 11.9
+    # the launch that also un-rotates gives what backward + Transform.backward give, bit for bit
+    quats, zeros = dev(c["quats"]), dev(np.zeros_like(c["centers"]))
+    two_calls = grads.clone()
+    mg.transform_batch(off, quats, dev(c["centers"]), zeros, two_calls, two_calls, dotranslate=False,
+                       inverse=True)
+    fused = torch.empty_like(grads)
+    gm.backward_batch(off, c["centers"], moved, types, radii, diff, fused,
+                      unrotate=(quats, dev(c["centers"])))
+    assert torch.equal(fused, two_calls)
     # linear in the upstream gradient: a factor of two is exact in floating point
     grads2 = torch.empty_like(grads)
     gm.backward_batch(off, c["centers"], moved, types, radii, diff * 2, grads2)
