@@ -60,7 +60,7 @@ def step_breakdown(fns, iters):
             for i in range(len(fns))]
 
 
-TRAFFIC_PROFILE = os.path.join("profiles", "bench_step_config1_kernel_trace.txt")
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_kernel_trace_and_traffic.txt")
 
 
 def measured_traffic(kernel):

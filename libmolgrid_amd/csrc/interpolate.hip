@@ -5,10 +5,13 @@
 // along z, so that its stores are whole 64-byte lines).  The tile maps to a rotated box in the
 // input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), marks the
 // window positions that some tap of the tile reads (about 40 % of the window: the rest of the
-// bounding box is never touched), deals those positions out evenly to its threads, and then stages
-// them one channel at a time into LDS (zero outside the input grid, so the taps need no bounds
-// tests); every thread reads its eight taps from LDS.  The source position, tap offsets and
-// weights are computed once per output voxel and reused for every channel.  Staging runs two
+// bounding box is never touched; a bit per position, one word per (x, y) row), numbers the marked
+// positions that lie inside the input grid in window order, and deals them out evenly to its
+// threads.  Per channel the threads stage those positions -- and nothing else -- into an LDS
+// buffer in that order (12 KB instead of the 39 KB of the whole window, so that four workgroups
+// share a CU), and every thread reads its eight taps from the slots it looked up once; a tap
+// outside the input grid reads a cell that holds zero.  The source position, the tap slots and
+// the weights are computed once per output voxel and reused for every channel.  Staging runs two
 // channels ahead of the interpolation: two register sets and two LDS buffers, one barrier per
 // channel.  Workgroups are numbered so that all tiles of one example run on the same XCD (they
 // share its input through that XCD's L2) and z-neighbouring tiles, which complete each other's
@@ -68,33 +71,44 @@ constexpr int kTileX = 8, kTileY = 8, kTileZ = 16;   // output tile; 16 voxels o
 constexpr int kTileThreads = 512;              // two output voxels (x and x + 4) per thread
 constexpr int kTileWaves = kTileThreads / 64;
 constexpr int kVox = kTileX * kTileY * kTileZ / kTileThreads;
-constexpr int kWin = 21;                       // largest staged window side
-constexpr int kWinZ = 22;                      // z stride of the window in LDS (even: 8-byte pairs)
-constexpr int kWinSize = kWin * kWin * kWinZ;  // floats per buffer
-constexpr int kFewRounds = 6;                  // staged elements per thread and channel (6 x 512 >= 2,800)
+constexpr int kWin = 21;                       // largest window side (the tile's bounding box in the input)
+constexpr int kRows = kWin * kWin;             // (x, y) rows of the window
+constexpr int kRowsPad = 448;
+constexpr int kFewRounds = 6;                  // staged elements per thread and channel
+constexpr int kSlots = kFewRounds * kTileThreads;   // 3,072 >= the 2,800 input voxels a tile can need
+constexpr int kBuf = kSlots + 4;               // floats per buffer: the slots and a cell that holds zero
 // longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
 constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
 
 __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     InterpArg p, int nbatch, int tiles_x, int tiles_z, Vec3Arg in_centers,
     const float* __restrict__ in, Vec4Arg quats, Vec3Arg rot_centers, Vec3Arg translations,
-    Vec3Arg out_centers, float* __restrict__ out, int plain_staging) {
-  extern __shared__ __align__(16) float s_win[];   // two buffers of kWinSize floats, one spare slot
+    Vec3Arg out_centers, float* __restrict__ out, int gather_only) {
+  // Two buffers of staged input values, in plan order (below).  While the plan is made the same
+  // memory holds its tables: per window row the z positions in use (a bit mask) and the row's
+  // first slot, then the list of source offsets.
+  __shared__ __align__(16) float s_buf[2 * kBuf];
   __shared__ float s_lo[3], s_hi[3];
   __shared__ int s_scan[kTileWaves];
+  unsigned* const s_rowmask = reinterpret_cast<unsigned*>(s_buf);
+  int* const s_rowstart = reinterpret_cast<int*>(s_buf) + kRowsPad;
+  int* const s_list = reinterpret_cast<int*>(s_buf) + 2 * kRowsPad;
+  static_assert(kBuf * 4 + 4 < 65536, "16-bit byte offsets");
+  static_assert(2 * kRowsPad + kSlots <= 2 * kBuf, "the plan's tables fit the buffers");
 
   // workgroup -> (example, tile): consecutive workgroups are dealt round-robin to the 8 XCDs, so
   // example b is pinned to XCD b % 8 and its tiles run there in z-fastest order
   const int tiles = tiles_x * tiles_x * tiles_z;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int b = (slot / tiles) * 8 + xcd;
+  const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
+  const int b = (slot_id / tiles) * 8 + xcd;
   if (b >= nbatch) return;
-  const int tile = slot % tiles;
+  const int tile = slot_id % tiles;
   const int tz = tile % tiles_z, ty = (tile / tiles_z) % tiles_x;
   const int tx = tile / (tiles_z * tiles_x);
 
   const int od = p.out_dim, id = p.in_dim;
   const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   // 16 consecutive lanes run along z: one store instruction writes whole 64-byte lines
   const int i0 = tx * kTileX + (tid >> 7), j = ty * kTileY + ((tid >> 4) & 7), k = tz * kTileZ + (tid & 15);
 
@@ -104,6 +118,7 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   const float4 qinvinv = quat_inverse(qinv);
 
   // ---- window of the tile: bounding box of the images of its eight corners -----------------
+  if (tid < kRowsPad) s_rowmask[tid] = 0u;
   if (tid < 8) {
     const int ci = min(tx * kTileX + ((tid >> 2) & 1) * (kTileX - 1), od - 1);
     const int cj = min(ty * kTileY + ((tid >> 1) & 1) * (kTileY - 1), od - 1);
@@ -138,8 +153,8 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   }
 
   // ---- this thread's taps and corner weights (channel independent) ---------------------------
-  int tap[kVox];
-  float cw[kVox][8];   // weight of tap (x, y, z) at index 4x + 2y + z
+  int wpos[kVox];      // window position of the low tap: (x * kWin + y) << 8 | z
+  float frac[kVox][3];   // fractional parts of the source position
   bool live[kVox];
 #pragma unroll
   for (int v = 0; v < kVox; ++v) {
@@ -150,63 +165,41 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     const float fx = floorf(s.gx), fy = floorf(s.gy), fz = floorf(s.gz);
     // fractional parts; an integral coordinate gives weight 0 to the upper tap
     const float xd = s.gx - fx, yd = s.gy - fy, zd = s.gz - fz;
-    const float x0 = 1.f - xd, y0 = 1.f - yd, z0 = 1.f - zd;
-    cw[v][0] = x0 * y0 * z0; cw[v][1] = x0 * y0 * zd; cw[v][2] = x0 * yd * z0; cw[v][3] = x0 * yd * zd;
-    cw[v][4] = xd * y0 * z0; cw[v][5] = xd * y0 * zd; cw[v][6] = xd * yd * z0; cw[v][7] = xd * yd * zd;
+    frac[v][0] = xd;
+    frac[v][1] = yd;
+    frac[v][2] = zd;
     // window-relative tap position, clamped into the window (a clamped tap is outside the input
     // grid on that side and its neighbours there are zero as well)
     const int wx = min(max((int)fminf(fmaxf(fx, -4.f), (float)id + 4.f) - wlo[0], 0), wn[0] - 2);
     const int wy = min(max((int)fminf(fmaxf(fy, -4.f), (float)id + 4.f) - wlo[1], 0), wn[1] - 2);
     const int wz = min(max((int)fminf(fmaxf(fz, -4.f), (float)id + 4.f) - wlo[2], 0), wn[2] - 2);
-    tap[v] = (wx * kWin + wy) * kWinZ + wz;
-  }
-
-  // ---- which window positions any voxel of the tile reads ------------------------------------
-  // The window is the bounding box of a rotated tile, so most of it is never touched.  One byte per
-  // window position (the window's own LDS, before it is first filled): every thread marks its
-  // sixteen taps.
-  {
-    unsigned char* used = reinterpret_cast<unsigned char*>(s_win);
-    unsigned* used4 = reinterpret_cast<unsigned*>(s_win);
-    for (int n = tid; n < (kWinSize + 3) / 4; n += kTileThreads) used4[n] = 0u;
-    __syncthreads();
-#pragma unroll
-    for (int v = 0; v < kVox; ++v) {
-      if (live[v]) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-          used[tap[v] + (c >> 2) * (kWin * kWinZ) + ((c >> 1) & 1) * kWinZ + (c & 1)] = 1;
-      }
+    wpos[v] = ((wx * kWin + wy) << 8) | wz;
+    // ---- which window positions any voxel of the tile reads: the window is the bounding box of a
+    // rotated tile, so most of it is never touched
+    if (live[v]) {
+      const unsigned bits = 3u << wz;
+      const int r = wx * kWin + wy;
+      atomicOr(&s_rowmask[r], bits);
+      atomicOr(&s_rowmask[r + 1], bits);
+      atomicOr(&s_rowmask[r + kWin], bits);
+      atomicOr(&s_rowmask[r + kWin + 1], bits);
     }
-    __syncthreads();
   }
+  __syncthreads();
 
-  // ---- staging plan: the window positions in use, in window order, dealt out evenly ------------
-  // Window positions outside the input grid hold zero for every channel: both buffers are cleared
-  // once and such positions, the positions no tap reads and the unused tail of a thread's share
-  // are steered to a spare LDS slot and to element 0 of the channel, so that the per-channel loop
-  // is load + write without tests.
-  // One thread per (x, y) row of the window (at most 21 x 21 of them) collects, as a bit mask,
-  // the z positions of its row that some tap reads and the input grid holds; a prefix sum over the
-  // workgroup numbers them in window order, so neighbouring slots are neighbouring addresses; the
-  // (source offset, LDS cell) pairs go to a list in the window's LDS and are read back strided by
-  // the workgroup size: every thread gets an equal share.
-  const int wcount = wn[0] * wn[1] * wn[2];
-  const int plane = wn[1] * wn[2];
-  const int lane = tid & 63, wave = tid >> 6;
+  // ---- staging plan: the window positions in use and inside the input grid, numbered in window
+  // order (row by row, z ascending): slot n of a buffer holds the n-th of them, and thread t stages
+  // slots t, t + 512, ...  One thread per row counts the row's positions, a prefix sum over the
+  // workgroup gives the row its first slot.
   unsigned zmask = 0;
-  int row_cell = 0, row_src = 0;
-  if (tid < wn[0] * wn[1]) {
-    const int ex = tid / wn[1], ey = tid - ex * wn[1];
+  int row_src = 0;
+  if (tid < kRows) {
+    const int ex = tid / kWin, ey = tid - ex * kWin;
     const int gx = wlo[0] + ex, gy = wlo[1] + ey;
-    row_cell = (ex * kWin + ey) * kWinZ;
     row_src = (gx * id + gy) * id + wlo[2];
-    if (gx >= 0 && gx < id && gy >= 0 && gy < id) {
-      const unsigned char* used = reinterpret_cast<const unsigned char*>(s_win) + row_cell;
-      for (int ez = 0; ez < wn[2]; ++ez) {
-        const int gz = wlo[2] + ez;
-        if (gz >= 0 && gz < id && used[ez] != 0) zmask |= 1u << ez;
-      }
+    if (ex < wn[0] && ey < wn[1] && gx >= 0 && gx < id && gy >= 0 && gy < id) {
+      const int zl = max(0, -wlo[2]), zh = min(wn[2], id - wlo[2]);   // z positions inside the grid
+      if (zh > zl) zmask = s_rowmask[tid] & ((1u << zh) - 1u) & ~((1u << zl) - 1u);
     }
   }
   const int mine = __popc(zmask);
@@ -217,182 +210,164 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     if (lane >= d) incl += up;
   }
   if (lane == 63) s_scan[wave] = incl;
-  __syncthreads();   // wave totals complete; every thread has read the marks
+  __syncthreads();   // wave totals complete; every row has read its marks
   int slot0 = incl - mine, planned = 0;
 #pragma unroll
   for (int w = 0; w < kTileWaves; ++w) {
-    const int c = s_scan[w];
-    slot0 += w < wave ? c : 0;
-    planned += c;
+    const int n = s_scan[w];
+    slot0 += w < wave ? n : 0;
+    planned += n;
   }
-  {
-    int* list = reinterpret_cast<int*>(s_win);             // pairs: source offset, destination
-    unsigned m = zmask;
-    int slot = slot0;
-    while (m != 0) {
-      const int ez = __builtin_ctz(m);
-      m &= m - 1u;
-      list[2 * slot] = row_src + ez;
-      list[2 * slot + 1] = row_cell + ez;
-      ++slot;
-    }
-  }
-  __syncthreads();
   const int rounds_used = (planned + kTileThreads - 1) / kTileThreads;   // uniform
-  int st_src[kFewRounds];   // offset inside one input channel
-  int st_dst[kFewRounds];   // offset inside the LDS window
-  {
-    const int* list = reinterpret_cast<const int*>(s_win);
-#pragma unroll
-    for (int e = 0; e < kFewRounds; ++e) {
-      const int slot = tid + e * kTileThreads;
-      const bool have = slot < planned;
-      st_src[e] = have ? list[2 * slot] : 0;
-      st_dst[e] = have ? list[2 * slot + 1] : 2 * kWinSize;
+  // (the buffer loads of the main path address one example's input with 32 bits)
+  const bool gather = rounds_used > kFewRounds || gather_only ||
+                      (size_t)p.channels * id * id * id * sizeof(float) >= 0x7fffffffull;
+  if (tid < kRows) {
+    s_rowmask[tid] = zmask;
+    s_rowstart[tid] = slot0;
+    if (!gather) {
+      unsigned m = zmask;
+      int slot = slot0;
+      while (m != 0) {
+        const int ez = __builtin_ctz(m);
+        m &= m - 1u;
+        s_list[slot++] = row_src + ez;
+      }
     }
-  }
-  __syncthreads();   // every thread holds its share: the window can be cleared
-  {
-    float4* z4 = reinterpret_cast<float4*>(s_win);
-    for (int n = tid; n < 2 * kWinSize / 4; n += kTileThreads) z4[n] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
   __syncthreads();
 
   const size_t in_chan = (size_t)id * id * id;
   const size_t out_points = (size_t)od * od * od;
   const float* src = in + (size_t)b * p.channels * in_chan;
-  float* dst = out + (size_t)b * p.channels * out_points + ((size_t)i0 * od + j) * od + k;
   const size_t vox_step = (size_t)(kTileX / kVox) * od * od;
-
-  // channel `ch` of the tile from the window buffer that holds it
-  auto interpolate_channel = [&](int ch, int which) {
-    const float* buf = s_win + which * kWinSize;
-#pragma unroll
-    for (int v = 0; v < kVox; ++v) {
-      const float* w = buf + tap[v];
-      float val = w[0] * cw[v][0];
-      val = fmaf(w[1], cw[v][1], val);
-      val = fmaf(w[kWinZ], cw[v][2], val);
-      val = fmaf(w[kWinZ + 1], cw[v][3], val);
-      val = fmaf(w[kWin * kWinZ], cw[v][4], val);
-      val = fmaf(w[kWin * kWinZ + 1], cw[v][5], val);
-      val = fmaf(w[kWin * kWinZ + kWinZ], cw[v][6], val);
-      val = fmaf(w[kWin * kWinZ + kWinZ + 1], cw[v][7], val);
-      if (live[v]) dst[(size_t)ch * out_points + v * vox_step] = val;
-    }
-  };
   const int C = p.channels;
 
-  if (rounds_used > kFewRounds || plain_staging) {
-    // More planned elements than the register sets below hold.  The launcher sends only resolution
-    // ratios here for which a tile needs at most 2,800 input voxels (the cells that meet the
-    // rotated 7 x 7 x 15 box grown by the taps), so this is a safety net: every thread copies
-    // whole-window elements straight into one buffer, working out the positions as it goes.
-    const float inv_plane_ = 1.0f / (float)plane, inv_row_ = 1.0f / (float)wn[2];
-    for (int ch = 0; ch < C; ++ch) {
-      const float* chan = src + (size_t)ch * in_chan;
-      for (int n = tid; n < wcount; n += kTileThreads) {
-        int ex = (int)((float)n * inv_plane_);
-        ex -= (ex * plane > n) ? 1 : 0;
-        ex += ((ex + 1) * plane <= n) ? 1 : 0;
-        const int r = n - ex * plane;
-        int ey = (int)((float)r * inv_row_);
-        ey -= (ey * wn[2] > r) ? 1 : 0;
-        ey += ((ey + 1) * wn[2] <= r) ? 1 : 0;
-        const int ez = r - ey * wn[2];
-        const int gx = wlo[0] + ex, gy = wlo[1] + ey, gz = wlo[2] + ez;
-        if (gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id)
-          s_win[(ex * kWin + ey) * kWinZ + ez] = chan[(gx * id + gy) * id + gz];
+  if (gather) {
+    // More positions than the buffers hold.  The launcher sends only resolution ratios here for
+    // which a tile needs at most 2,800 input voxels, so this is a safety net (and a test hook):
+    // every thread gathers its taps from global memory, with the weights and the order of the
+    // sums of the main path.
+    float* dst = out + (size_t)b * C * out_points + ((size_t)i0 * od + j) * od + k;
+#pragma unroll
+    for (int v = 0; v < kVox; ++v) {
+      if (!live[v]) continue;
+      const int wx = (wpos[v] >> 8) / kWin, wy = (wpos[v] >> 8) - wx * kWin, wz = wpos[v] & 255;
+      int o[8];
+      bool ok[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int gx = wlo[0] + wx + (q >> 2), gy = wlo[1] + wy + ((q >> 1) & 1), gz = wlo[2] + wz + (q & 1);
+        ok[q] = gx >= 0 && gx < id && gy >= 0 && gy < id && gz >= 0 && gz < id;
+        o[q] = ok[q] ? (gx * id + gy) * id + gz : 0;
       }
-      __syncthreads();
-      interpolate_channel(ch, 0);
-      __syncthreads();
+      for (int ch = 0; ch < C; ++ch) {
+        const float* chan = src + (size_t)ch * in_chan;
+        float t8[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) t8[q] = ok[q] ? chan[o[q]] : 0.f;
+        dst[(size_t)ch * out_points + v * vox_step] =
+            lerp3(t8[0], t8[1], t8[2], t8[3], t8[4], t8[5], t8[6], t8[7], frac[v][0], frac[v][1], frac[v][2]);
+      }
     }
     return;
   }
+
+  // ---- slots of this thread's taps (byte offsets inside a buffer; the zero cell for a tap that
+  // lies outside the input grid), and the sources of the slots it stages
+  unsigned tap_off[kVox][4];   // two 16-bit byte offsets each: the taps at z and z + 1
+#pragma unroll
+  for (int v = 0; v < kVox; ++v) {
+    const int r0 = wpos[v] >> 8, wz = wpos[v] & 255;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = r0 + (q >> 1) * kWin + (q & 1);
+      const unsigned m = s_rowmask[r];
+      const int first = s_rowstart[r];
+      unsigned both = 0;
+#pragma unroll
+      for (int dz = 0; dz < 2; ++dz) {
+        const int bit = wz + dz;
+        const bool have = (m >> bit) & 1u;
+        const int slot = first + __popc(m & ((1u << bit) - 1u));
+        both |= ((unsigned)(have ? slot : kSlots) * 4u) << (16 * dz);
+      }
+      tap_off[v][q] = both;
+    }
+  }
+  int st_src[kFewRounds];   // byte offset inside one input channel
+#pragma unroll
+  for (int e = 0; e < kFewRounds; ++e) {
+    const int slot = tid + e * kTileThreads;
+    st_src[e] = (slot < planned ? s_list[slot] : 0) * 4;   // a slot past the plan is read by no tap
+  }
+  __syncthreads();   // the tables have been read: the buffers can be filled
+  if (tid == 0) s_buf[kSlots] = s_buf[kBuf + kSlots] = 0.f;
 
   // Two register sets, so that the loads of a channel are issued a whole channel before they are
   // needed: while channel ch is interpolated from one buffer, channel ch + 1 is written to the
   // other and channel ch + 2 is in flight.  Every load and store of the loop is issued
-  // unconditionally -- unused staging slots read element 0 into a spare LDS cell, voxels outside
-  // the output grid store through a buffer descriptor to an offset past its end, which the
-  // hardware drops -- because loads and stores share one in-order counter: only with a fixed
-  // number of them per iteration can a wait for channel ch + 1 leave the loads of channel ch + 2
-  // and the stores of channel ch in flight.
+  // unconditionally -- slots past the plan stage element 0, voxels outside the output grid store
+  // through a buffer descriptor to an offset past its end, which the hardware drops -- because
+  // loads and stores share one in-order counter: only with a fixed number of them per iteration
+  // can a wait for channel ch + 1 leave the loads of channel ch + 2 and the stores of channel ch
+  // in flight.
   float ra[kFewRounds], rb[kFewRounds];
+  // (buffer loads: the channel's offset is a scalar operand, the slot's source a 32-bit offset)
+  const __amdgpu_buffer_rsrc_t in_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(src), 0, (int)((size_t)C * in_chan * sizeof(float)), 0x00020000);
   auto fetch = [&](float (&r)[kFewRounds], int ch) {
-    const float* chan = src + (size_t)ch * in_chan;
-#pragma unroll
-    for (int e = 0; e < kFewRounds; ++e) r[e] = chan[st_src[e]];
-  };
-  auto deposit = [&](const float (&r)[kFewRounds], int ch) {
-    const int base = (ch & 1) * kWinSize;
-#pragma unroll
-    for (int e = 0; e < kFewRounds; ++e)   // (the spare slot is the same for both buffers)
-      s_win[st_dst[e] == 2 * kWinSize ? 2 * kWinSize : base + st_dst[e]] = r[e];
-  };
-  const size_t out_bytes = (size_t)C * out_points * sizeof(float);
-  if (out_bytes < 0x7fffffffull) {
-    const __amdgpu_buffer_rsrc_t out_buf = __builtin_amdgcn_make_buffer_rsrc(
-        out + (size_t)b * C * out_points, 0, (int)out_bytes, 0x00020000);
-    unsigned off[kVox];
-#pragma unroll
-    for (int v = 0; v < kVox; ++v)
-      off[v] = live[v] ? (unsigned)((((size_t)i0 * od + j) * od + k + v * vox_step) * sizeof(float))
-                       : (unsigned)out_bytes;            // past the end for every channel
-    auto interpolate_buffered = [&](int ch, int which) {
-      const float* buf = s_win + which * kWinSize;
-      const unsigned chan_off = (unsigned)((size_t)ch * out_points * sizeof(float));
-#pragma unroll
-      for (int v = 0; v < kVox; ++v) {
-        const float* w = buf + tap[v];
-        float val = w[0] * cw[v][0];
-        val = fmaf(w[1], cw[v][1], val);
-        val = fmaf(w[kWinZ], cw[v][2], val);
-        val = fmaf(w[kWinZ + 1], cw[v][3], val);
-        val = fmaf(w[kWin * kWinZ], cw[v][4], val);
-        val = fmaf(w[kWin * kWinZ + 1], cw[v][5], val);
-        val = fmaf(w[kWin * kWinZ + kWinZ], cw[v][6], val);
-        val = fmaf(w[kWin * kWinZ + kWinZ + 1], cw[v][7], val);
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), out_buf,
-                                              (int)(off[v] + chan_off), 0, 0);
-      }
-    };
-    fetch(ra, 0);
-    deposit(ra, 0);
-    fetch(ra, C > 1 ? 1 : 0);
-    __syncthreads();
-    for (int ch = 0; ch < C; ch += 2) {
-      fetch(rb, ch + 2 < C ? ch + 2 : ch);
-      if (ch + 1 < C) deposit(ra, ch + 1);
-      interpolate_buffered(ch, 0);
-      __syncthreads();
-      if (ch + 1 >= C) break;
-      fetch(ra, ch + 3 < C ? ch + 3 : ch);
-      if (ch + 2 < C) deposit(rb, ch + 2);
-      interpolate_buffered(ch + 1, 1);
-      __syncthreads();
-    }
-    return;
-  }
-  // grids of 2 GB or more per example: plain stores under their conditions
-  auto fetch_some = [&](float (&r)[kFewRounds], int ch) {
-    const float* chan = src + (size_t)ch * in_chan;
+    const int chan_off = __builtin_amdgcn_readfirstlane((int)((size_t)ch * in_chan * sizeof(float)));
 #pragma unroll
     for (int e = 0; e < kFewRounds; ++e)
-      if (e < rounds_used) r[e] = chan[st_src[e]];
+      r[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(in_buf, st_src[e], chan_off, 0));
   };
-  fetch_some(ra, 0);
+  auto deposit = [&](const float (&r)[kFewRounds], int ch) {
+    float* buf = s_buf + (ch & 1) * kBuf + tid;
+#pragma unroll
+    for (int e = 0; e < kFewRounds; ++e) buf[e * kTileThreads] = r[e];
+  };
+  const size_t out_bytes = (size_t)C * out_points * sizeof(float);
+  const bool buffered = out_bytes < 0x7fffffffull;
+  const __amdgpu_buffer_rsrc_t out_buf = __builtin_amdgcn_make_buffer_rsrc(
+      out + (size_t)b * C * out_points, 0, buffered ? (int)out_bytes : 0, 0x00020000);
+  float* const dst = out + (size_t)b * C * out_points + ((size_t)i0 * od + j) * od + k;
+  unsigned off[kVox];
+#pragma unroll
+  for (int v = 0; v < kVox; ++v)
+    off[v] = live[v] ? (unsigned)((((size_t)i0 * od + j) * od + k + v * vox_step) * sizeof(float))
+                     : (unsigned)out_bytes;            // past the end for every channel
+  auto interpolate_channel = [&](int ch, int which) {
+    const char* buf = reinterpret_cast<const char*>(s_buf + which * kBuf);
+    const unsigned chan_off = (unsigned)((size_t)ch * out_points * sizeof(float));
+#pragma unroll
+    for (int v = 0; v < kVox; ++v) {
+      float t8[8];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        t8[2 * q] = *reinterpret_cast<const float*>(buf + (tap_off[v][q] & 0xffffu));
+        t8[2 * q + 1] = *reinterpret_cast<const float*>(buf + (tap_off[v][q] >> 16));
+      }
+      const float val = lerp3(t8[0], t8[1], t8[2], t8[3], t8[4], t8[5], t8[6], t8[7], frac[v][0],
+                              frac[v][1], frac[v][2]);
+      if (buffered)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), out_buf,
+                                              (int)(off[v] + chan_off), 0, 0);
+      else if (live[v])   // grids of 2 GB or more per example
+        dst[(size_t)ch * out_points + v * vox_step] = val;
+    }
+  };
+  fetch(ra, 0);
   deposit(ra, 0);
-  if (C > 1) fetch_some(ra, 1);
+  fetch(ra, C > 1 ? 1 : 0);
   __syncthreads();
   for (int ch = 0; ch < C; ch += 2) {
-    if (ch + 2 < C) fetch_some(rb, ch + 2);
+    fetch(rb, ch + 2 < C ? ch + 2 : ch);
     if (ch + 1 < C) deposit(ra, ch + 1);
     interpolate_channel(ch, 0);
     __syncthreads();
     if (ch + 1 >= C) break;
-    if (ch + 3 < C) fetch_some(ra, ch + 3);
+    fetch(ra, ch + 3 < C ? ch + 3 : ch);
     if (ch + 2 < C) deposit(rb, ch + 2);
     interpolate_channel(ch + 1, 1);
     __syncthreads();
@@ -472,16 +447,12 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
     const int tiles_z = (p.out_dim + kTileZ - 1) / kTileZ;
     const int tiles = tiles_x * tiles_x * tiles_z;
     const int groups = (nbatch + 7) / 8;
-    const size_t lds = (2 * (size_t)kWinSize + 4) * sizeof(float);   // two buffers and a spare slot
-    // test hook: take the plain staging path (otherwise only a safety net) for every tile
+    // test hook: every tile takes the gather path (otherwise only a safety net)
     const char* hook = getenv("MOLGRID_HIP_INTERP_PLAIN_STAGING");
-    const int plain_staging = (hook != nullptr && hook[0] == '1') ? 1 : 0;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(interpolate_tiled_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), lds,
+    const int gather_only = (hook != nullptr && hook[0] == '1') ? 1 : 0;
+    hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), 0,
                        stream, p, nbatch, tiles_x, tiles_z, in_centers, in, quats, rot_centers,
-                       translations, out_centers, out, plain_staging);
+                       translations, out_centers, out, gather_only);
     return hipGetLastError();
   }
   const int out_points = p.out_dim * p.out_dim * p.out_dim;
