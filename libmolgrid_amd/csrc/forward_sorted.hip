@@ -3,7 +3,8 @@
 //
 // 1. sort_atoms_kernel: the atoms of every example become 16-byte records (x, y, z, ar =
 //    radius * radius_scale), sorted by (channel, x slab of the centre) and, within a key, in
-//    ascending atom order (a stable counting sort, one workgroup per example).  Atoms without a
+//    ascending atom order (a stable counting sort, one workgroup per example and group of a few
+//    channels).  Atoms without a
 //    channel drop out.  The workgroup also finds the rank of its example by size and writes the
 //    example's tables -- grid origin, example number, and for every (channel, x slab) the run of
 //    records that can reach the slab -- at that rank, so that the second launch meets the examples
@@ -27,7 +28,6 @@
 // Every global access of the splat kernel goes through buffer instructions that carry the
 // extent of the array they address: an index outside it reads zero or is dropped.
 #include <algorithm>
-#include <cstdlib>
 
 #include "kernels.h"
 #include "splat_common.h"
@@ -617,11 +617,6 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
   }
 }
 
-int exp_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : fallback;
-}
-
 template <bool BINARY, bool EXACT, int COLS>
 hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, float* out,
                         hipStream_t stream) {
@@ -629,10 +624,8 @@ hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, floa
   const int nxs = (dim + kColXY - 1) / kColXY;
   const int nyp = (dim + kColXY * COLS - 1) / (kColXY * COLS);
   const int nzs = (dim + kSlabZ - 1) / kSlabZ;
-  static const int exp_ranges = exp_int("MOLGRID_EXP_RANGES", 0);
-  int nranges = std::max((g.ntypes + kItemChannels - 1) / kItemChannels,
-                         (g.ntypes + kItemChannelsMax - 1) / kItemChannelsMax);
-  if (exp_ranges) nranges = std::max(exp_ranges, (g.ntypes + kItemChannelsMax - 1) / kItemChannelsMax);
+  const int nranges = std::max((g.ntypes + kItemChannels - 1) / kItemChannels,
+                               (g.ntypes + kItemChannelsMax - 1) / kItemChannelsMax);
   const long long nitems = (long long)nbatch * nxs * nzs * nyp * nranges;
   if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
   const int aligned = ((dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
@@ -677,13 +670,11 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
 
-  static const int cols = exp_int("MOLGRID_EXP_MODE", 0) & 3;          // 0: two columns, 1: one
   if (exact) {
     if (binary) return launch_splat<true, true, 1>(g, s, nbatch, out, stream);
     return launch_splat<false, true, 1>(g, s, nbatch, out, stream);
   }
   if (binary) return launch_splat<true, false, 2>(g, s, nbatch, out, stream);
-  if (cols == 1) return launch_splat<false, false, 1>(g, s, nbatch, out, stream);
   return launch_splat<false, false, 2>(g, s, nbatch, out, stream);
 }
 

@@ -3,26 +3,36 @@
 //
 // Every atom feeds every channel: out[c][v] = sum_a W[a][c] * D[a][v] with W the type vector of
 // atom a and D its density at voxel v.  That is a matrix product, and the only dense contraction of
-// the gridding path, so it runs on the matrix cores: v_mfma_f32_16x16x4f32 multiplies a
-// 16-channel x 4-atom slice of W with a 4-atom x 16-voxel slice of D into a 16 x 16 tile of sums
-// (all float32).  The VALU evaluates each density once; the 28 multiply-adds per atom and voxel of
-// a plain loop are gone.
+// the gridding path: v_mfma_f32_16x16x4f32 multiplies a 16-channel x 4-atom slice of W with a
+// 4-atom x 16-voxel slice of D into a 16 x 16 tile of sums (all float32).  The VALU evaluates
+// each density once; the 28 multiply-adds per atom and voxel of a plain loop become two matrix
+// instructions per four atoms and 64 voxels.  On this chip a float32 matrix instruction and VALU
+// work do not overlap on a SIMD (a loop of eight such instructions and 64 independent v_fma_f32
+// takes the sum of the two loops' times, with one, two or three waves on the SIMD), so the kernel
+// is bound by the sum of the two, not by the larger.
 //
-// Geometry, culling and write-out follow the column kernel of forward_index.hip: a workgroup (four
-// waves) owns a group of three columns of 4 x 4 voxels in (x, y) over a slab of up to 48 voxels in z
-// and takes them one after the other; the atoms that can reach the group are found by one scan and
-// kept as indices, records (x, y, z, 1/ar^2, atom) are built 256 at a time, each wave culls them
-// again per 4x4x4 block into a private list, and the sums leave through a double-buffered LDS stage
-// as float4 pieces of whole z rows.  A wave keeps the 32 x 64 sums of each of its three blocks in
-// eight 4-register tiles: two halves of the channels by the four x planes of the 4x4x4 voxels.
+// A workgroup (four waves) owns a group of three columns of 4 x 4 voxels in (x, y) over a slab of
+// up to 48 voxels in z and takes the columns one after the other; a wave owns three 4x4x4 blocks
+// of the column.  The atoms that can reach the group are found by one scan and kept as indices.
+// For a column they are taken 256 at a time: the workgroup builds a row per atom in LDS -- its 32
+// weights of the pass (zero past the last channel) and its record (x, y, z, 1/ar^2) -- each wave
+// culls the rows against its three blocks in one pass (the x and y terms of the box distance are
+// shared) into three lists of row offsets, and then walks each list four atoms a step.  The walk
+// is software-pipelined two steps a trip: rows and list entries are read ahead, the densities of
+// the next step are evaluated between the matrix instructions of this one.  A list ends in
+// entries that point at a row of no atom (zero weights, unreachable record), so a short last
+// step and the read-ahead need no masks.  A wave keeps the 32 x 64 sums of each of its three
+// blocks in eight 4-register tiles: two halves of the channels by the four x planes of the block.
+// The sums leave through an LDS stage, eight channels a round with every lane writing, as float4
+// pieces of whole z rows.
 //
 // Binary occupancy adds the weights themselves (density 1 where the atom covers the voxel, by the
 // reference's exact float comparison) and is compared bit for bit with the CPU loop, which adds
 // them in atom order.  v_mfma_f32_16x16x4f32 adds the four products of a step to the running sum
 // one after the other, each rounded to float32 -- measured: every binary comparison of the test
-// suite (sums of tens of weights in tens of thousands of voxels) is identical -- so the order of
-// the list, ascending atoms, is the order of the sum.  Densities differ from the column kernel in
-// the last bits only because dy^2 + dz^2 is shared by the four x planes here.
+// suite (sums of tens of weights in up to 25 million voxels, full size included) is identical --
+// so the order of the list, ascending atoms, is the order of the sum.  Gaussian densities share
+// dy^2 + dz^2 between the four x planes and agree with the CPU loop to rounding.
 #include <type_traits>
 
 #include "kernels.h"
@@ -39,12 +49,16 @@ constexpr int kBlocksPerWave = 3;
 constexpr int kSlabZ = kColWaves * kBlocksPerWave * 4;   // 48
 constexpr int kRowPad = 52;                      // staged z row, padded against bank conflicts
 constexpr int kPlane = 16 * kRowPad;             // one staged channel: 16 rows
-constexpr int kStageCh = 4;                      // channels staged per round
+constexpr int kStageCh = 4;                      // channel planes a pass of the write-out covers
+constexpr int kPlaneS = kPlane + 4;              // stage plane stride: the four quads of a wave, which
+                                                 // write planes 2 apart, then meet no bank twice over
 constexpr int kSuper = 4096;                     // atoms scanned per pass
 constexpr int kSeg = kSuper / kColWaves;
 constexpr int kRecChunk = 256;
 constexpr int kChannels = 32;                    // channels per pass: the rows of a tile
-constexpr int kEntryBytes = 80;                  // four records (16 B each) and their four atoms
+constexpr int kRowBytes = 144;                   // a chunk row: 32 weights, then x, y, z, 1/ar^2
+constexpr int kStageBytes = 2 * kStageCh * kPlaneS * 4;
+constexpr int kRowsBytes = (kRecChunk + 1) * kRowBytes;   // the last row belongs to no atom
 
 
 __device__ __forceinline__ float uniform(float v) {
@@ -59,15 +73,18 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_waves_per_eu(3, 
 splat_vector_mfma_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_vector, const float* __restrict__ radii,
-    float* __restrict__ out, int cols_per_side, int vec_store) {
+    float* __restrict__ out, int cols_per_side, int vec_store, int vec_weights) {
   __shared__ unsigned short s_idx[kColWaves][kSeg];
   __shared__ int s_wcount[kColWaves];
-  __shared__ float4 s_rec[kRecChunk];            // x, y, z, 1/ar^2
-  __shared__ int s_recatom[kRecChunk];
-  // wave-private list of a block's atoms, four per entry; spare entries because the loop reads
-  // ahead
-  __shared__ __align__(16) unsigned char s_mini[kColWaves][(kWave / 4 + 3) * kEntryBytes];
-  __shared__ __align__(16) float s_stage[2 * kStageCh * kPlane];
+  // The rows of the current chunk of records while sums are formed, the stage of the write-out
+  // afterwards.  A row holds the atom's weights for the 32 channels of the pass (zero past the
+  // last channel) and its record; the row after the chunk has zero weights and a record at an
+  // unreachable distance, and lies past the stage, which never overwrites it.
+  __shared__ __align__(16) unsigned char s_rows[kRowsBytes > kStageBytes ? kRowsBytes : kStageBytes];
+  // wave-private lists of the atoms of each block (byte offsets of their rows); spare entries
+  // because the loop reads ahead
+  __shared__ unsigned short s_mini[kColWaves][kBlocksPerWave][kRecChunk + 24];
+  float* const s_stage = reinterpret_cast<float*>(s_rows);
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -159,26 +176,61 @@ splat_vector_mfma_kernel(
   };
 
   // ---- records: candidates [c0, c0 + m) of the current scan -----------------------------------
-  auto build_records = [&](int s0, int c0, int m) {
+  auto build_records = [&](int s0, int c0, int m, int cbase, int nchan) {
     if (tid < m) {
       const int gi = c0 + tid;
       int w = 0;
 #pragma unroll
       for (int k = 1; k < kColWaves; ++k) w += (gi >= segstart[k]) ? 1 : 0;
       const int a = s0 + s_idx[w][min(gi - segstart[w], kSeg - 1)];
+      const float* __restrict__ wrow = type_vector + (size_t)a * ntypes + cbase;
+      unsigned char* row = s_rows + tid * kRowBytes;
+      // the weights, four quads in flight at a time (the sums of the column stay in registers)
+#pragma unroll
+      for (int q0 = 0; q0 < kChannels / 4; q0 += 4) {
+        v4f wq[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = 4 * (q0 + u);
+          if (vec_weights) {
+            wq[u] = *reinterpret_cast<const v4f*>(wrow + min(c, nchan - 4));
+          } else {
+            wq[u].x = wrow[min(c, nchan - 1)];
+            wq[u].y = wrow[min(c + 1, nchan - 1)];
+            wq[u].z = wrow[min(c + 2, nchan - 1)];
+            wq[u].w = wrow[min(c + 3, nchan - 1)];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = 4 * (q0 + u);
+          v4f v = wq[u];
+          if (c >= nchan) v.x = 0.f;
+          if (c + 1 >= nchan) v.y = 0.f;
+          if (c + 2 >= nchan) v.z = 0.f;
+          if (c + 3 >= nchan) v.w = 0.f;
+          *reinterpret_cast<v4f*>(row + 4 * c) = v;
+        }
+      }
       float ar, ar2;
       {
 #pragma clang fp contract(off)
         ar = radii[a] * g.radius_scale;
         ar2 = ar * ar;
       }
-      s_rec[tid] = make_float4(coords[3 * a], coords[3 * a + 1], coords[3 * a + 2],
-                               BINARY ? ar2 : 1.0f / ar2);
-      s_recatom[tid] = a;
+      const v4f rec = {coords[3 * a], coords[3 * a + 1], coords[3 * a + 2], BINARY ? ar2 : 1.0f / ar2};
+      *reinterpret_cast<v4f*>(row + 4 * kChannels) = rec;
     }
     __syncthreads();
   };
 
+  // the row of no atom: zero weights, and a record no voxel is within reach of (its squared
+  // distance overflows to infinity, which passes neither comparison)
+  if (tid < kRowBytes / 4) {
+    float v = 0.f;
+    if (tid >= kChannels) v = tid < kChannels + 3 ? 1e30f : (BINARY ? -1.0f : 1.0f);
+    reinterpret_cast<float*>(s_rows + kRecChunk * kRowBytes)[tid] = v;
+  }
   // whole example in one scan when its survivors fit; else passes of kSuper atoms per column
   bool one_pass = false;
   if (end - begin <= 65536) one_pass = scan(begin, end);
@@ -190,11 +242,7 @@ splat_vector_mfma_kernel(
 
   for (int cbase = 0; cbase < ntypes; cbase += kChannels) {
     const int nchan = min(kChannels, ntypes - cbase);
-    // this lane's two rows of the weight matrix: channels cbase + j and cbase + 16 + j of every
-    // atom (a row past the last channel reads the last channel and is zeroed afterwards)
-    const bool chan_live[2] = {j < nchan, 16 + j < nchan};
-    const float* __restrict__ weights0 = type_vector + cbase + min(j, nchan - 1);
-    const float* __restrict__ weights1 = type_vector + cbase + min(16 + j, nchan - 1);
+    // (a lane's two rows of the weight matrix are channels cbase + j and cbase + 16 + j)
     for (int col = 0; col < kColsPerGroup; ++col) {
       const int y0 = gy0 + col * kColXY;
       if (y0 >= dim) break;
@@ -215,159 +263,180 @@ splat_vector_mfma_kernel(
         if (!one_pass) scan(s0, min(end, s0 + kSuper));
         for (int c0 = 0; c0 < ncand; c0 += kRecChunk) {
           const int m = min(kRecChunk, ncand - c0);
-          build_records(s0, c0, m);
+          build_records(s0, c0, m, cbase, nchan);
+          // one pass over the chunk's records finds, for each of the wave's blocks, the atoms
+          // that can reach it (the x and y terms of the box distance are shared); each list
+          // ends in rows of no atom, because the last step may be short and the loop reads one
+          // step ahead
+          int nlist[kBlocksPerWave];
+#pragma unroll
+          for (int blk = 0; blk < kBlocksPerWave; ++blk) nlist[blk] = 0;
+          for (int r0 = 0; r0 < m; r0 += kWave) {
+            const int i = min(r0 + lane, m - 1);
+            const float4 rec = *reinterpret_cast<const float4*>(s_rows + i * kRowBytes + 4 * kChannels);
+            const float ex = fmaxf(fmaxf(clx - rec.x, rec.x - chx), 0.f);
+            const float ey = fmaxf(fmaxf(cly - rec.y, rec.y - chy), 0.f);
+            const float exy = ex * ex + ey * ey;
+#pragma unroll
+            for (int blk = 0; blk < kBlocksPerWave; ++blk) {
+              const int zb = z0 + (wave * kBlocksPerWave + blk) * 4;
+              const float blz = uniform(grid_coord(oz, zb, g.resolution));
+              const float bhz = uniform(grid_coord(oz, min(zb + 4, zend) - 1, g.resolution));
+              const float ez = fmaxf(fmaxf(blz - rec.z, rec.z - bhz), 0.f);
+              const float d2 = exy + ez * ez;
+              const bool pass = (r0 + lane < m) && (zb < zend) &&
+                                (BINARY ? (d2 <= rec.w * kCullSlack) : (d2 * rec.w <= frm2 * kCullSlack));
+              const unsigned long long bm = __ballot(pass);
+              if (pass)
+                s_mini[wave][blk][nlist[blk] + __popcll(bm & ((1ull << lane) - 1ull))] =
+                    (unsigned short)(i * kRowBytes);
+              nlist[blk] += __popcll(bm);
+            }
+          }
+#pragma unroll
+          for (int blk = 0; blk < kBlocksPerWave; ++blk)
+            if (lane < 24) s_mini[wave][blk][nlist[blk] + lane] = (unsigned short)(kRecChunk * kRowBytes);
+
 #pragma unroll
           for (int blk = 0; blk < kBlocksPerWave; ++blk) {
+            const int n = nlist[blk];
+            if (n == 0) continue;
             const int zb = z0 + (wave * kBlocksPerWave + blk) * 4;
-            if (zb >= zend) continue;
-            const float blz = uniform(grid_coord(oz, zb, g.resolution));
-            const float bhz = uniform(grid_coord(oz, min(zb + 4, zend) - 1, g.resolution));
             // a voxel outside the grid sits at infinity: no atom reaches it
             const float vz = (y_live && zb + jz < zend) ? grid_coord(oz, zb + jz, g.resolution)
                                                         : INFINITY;
-            for (int r0 = 0; r0 < m; r0 += kWave) {
-              const int i = r0 + lane;
-              bool pass = false;
-              float4 rec = make_float4(0.f, 0.f, 0.f, 0.f);
-              if (i < m) {
-                rec = s_rec[i];
-                const float d2 = box_distance2(rec.x, rec.y, rec.z, clx, cly, blz, chx, chy, bhz);
-                pass = BINARY ? (d2 <= rec.w * kCullSlack) : (d2 * rec.w <= frm2 * kCullSlack);
-              }
-              const unsigned long long bm = __ballot(pass);
-              const int n = __popcll(bm);
-              if (n == 0) continue;
-              unsigned char* mine = s_mini[wave];
-              if (pass) {
-                const int p = __popcll(bm & ((1ull << lane) - 1ull));
-                unsigned char* e = mine + (p >> 2) * kEntryBytes;
-                *reinterpret_cast<float4*>(e + (p & 3) * 16) = rec;
-                *reinterpret_cast<int*>(e + 64 + (p & 3) * 4) = s_recatom[i];
-              }
-              // one entry = four atoms = one step of the matrix product; the quarter wave that
-              // holds atom `quad` reads its record and its two weights, every lane evaluates four
-              // densities (its (y, z) in each of the four x planes)
-              struct Step { float4 r; float w0, w1; bool have; };
-              auto fetch = [&](int k) -> Step {
-                const unsigned char* e = mine + k * kEntryBytes;
-                Step s;
-                s.r = *reinterpret_cast<const float4*>(e + quad * 16);
-                const int atom = *reinterpret_cast<const int*>(e + 64 + quad * 4);
-                s.have = 4 * k + quad < n;   // (past the list: an older atom or none)
-                // Both weights are always loaded (from the example's first atom where there is
-                // none) and masked only when they are used, an iteration later: the loads of
-                // the next entry then stay in flight while this entry is evaluated.
-                const size_t row = (size_t)(s.have ? atom : begin) * ntypes;
-                s.w0 = weights0[row];
-                s.w1 = weights1[row];
-                return s;
-              };
-              const int steps = (n + 3) >> 2;
-              Step cur = fetch(0);
-              for (int k = 0; k < steps; ++k) {
-                const Step nxt = fetch(k + 1);   // in flight while this entry is evaluated
-                __builtin_amdgcn_sched_barrier(0);  // (keeps the loads up here)
-                // a slot past the list has no reach at all, so its density is exactly zero (zero
-                // weight alone would not do: a stale record can give an infinite density, and
-                // 0 * inf is not a number)
-                const float rw = cur.have ? cur.r.w : (BINARY ? -1.0f : INFINITY);
-                const float w0 = (cur.have && chan_live[0]) ? cur.w0 : 0.f;
-                const float w1 = (cur.have && chan_live[1]) ? cur.w1 : 0.f;
-                const float dy = vy - cur.r.y, dz = vz - cur.r.z;
-                const float dyz2 = dy * dy + dz * dz;
+            const unsigned short* mine = s_mini[wave][blk];
+            // four atoms = one step of the matrix product; the quarter wave that holds atom
+            // `quad` reads its record and its two weights, every lane evaluates four densities
+            // (its (y, z) in each of the four x planes)
+            struct Step { float4 r; float w0, w1; };
+            auto fetch_row = [&](unsigned off) -> Step {
+              const unsigned char* row = s_rows + off;
+              Step s;
+              s.r = *reinterpret_cast<const float4*>(row + 4 * kChannels);
+              s.w0 = *reinterpret_cast<const float*>(row + 4 * j);
+              s.w1 = *reinterpret_cast<const float*>(row + 4 * (16 + j));
+              return s;
+            };
+            // the four densities of a lane for one atom: its (y, z) in each of the four x planes
+            auto densities = [&](const float4& r, float (&d)[4]) {
+              const float dy = vy - r.y, dz = vz - r.z;
+              const float dyz2 = dy * dy + dz * dz;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                  const float dx = vx[t] - cur.r.x;
-                  float d;
-                  if (BINARY) {
-                    // the reference's own float sequence ((dx^2 + dy^2) + dz^2) < ar^2
-                    d = sq_distance_exact(dx, dy, dz) < rw ? 1.0f : 0.0f;
-                  } else {
-                    const float u = (dx * dx + dyz2) * rw;
-                    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
-                    const float su = __builtin_amdgcn_sqrtf(u);
-                    const float quadr = fmaxf(fmaf(g.A, u, fmaf(g.B, su, g.C)), 0.f);
-                    d = (u <= grm2) ? gauss : quadr;
-                    d = (u <= frm2) ? d : 0.f;
-                  }
-                  sums[blk][t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w0, d, sums[blk][t][0], 0, 0, 0);
-                  sums[blk][t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w1, d, sums[blk][t][1], 0, 0, 0);
+              for (int t = 0; t < 4; ++t) {
+                const float dx = vx[t] - r.x;
+                if (BINARY) {
+                  // the reference's own float sequence ((dx^2 + dy^2) + dz^2) < ar^2
+                  d[t] = sq_distance_exact(dx, dy, dz) < r.w ? 1.0f : 0.0f;
+                } else {
+                  const float u = (dx * dx + dyz2) * r.w;
+                  const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                  const float su = __builtin_amdgcn_sqrtf(u);
+                  const float quadr = fmaxf(fmaf(g.A, u, fmaf(g.B, su, g.C)), 0.f);
+                  const float core = (u <= grm2) ? gauss : quadr;
+                  d[t] = (u <= frm2) ? core : 0.f;
                 }
-                cur = nxt;
               }
+            };
+            auto multiply = [&](const Step& s, const float (&d)[4]) {
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                sums[blk][t][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(s.w0, d[t], sums[blk][t][0], 0, 0, 0);
+                sums[blk][t][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(s.w1, d[t], sums[blk][t][1], 0, 0, 0);
+              }
+            };
+            // Two steps per trip, software-pipelined: while the matrix cores multiply the
+            // densities of one step, the VALU evaluates those of the next and the rows of the
+            // step after that are on their way from LDS.  The rows of no atom at the end of the
+            // list make a step past the last atom add nothing.
+            const int trips = (n + 7) >> 3;
+            Step a = fetch_row(mine[quad]);
+            Step b = fetch_row(mine[4 + quad]);
+            unsigned oc = mine[8 + quad], oe = mine[12 + quad];   // list entries, a trip ahead
+            float da[4], db[4];
+            densities(a.r, da);
+            for (int k = 0; k < 2 * trips; k += 2) {
+              const Step c = fetch_row(oc);
+              const Step e = fetch_row(oe);
+              oc = mine[4 * (k + 4) + quad];
+              oe = mine[4 * (k + 5) + quad];
+              multiply(a, da);
+              densities(b.r, db);
+              multiply(b, db);
+              densities(c.r, da);
+              a = c;
+              b = e;
             }
           }
           lds_barrier();   // records are rebuilt next round
         }
       }
 
-      // ---- store: four channels per round through a double-buffered LDS stage ----
-      int st_lds[kPer], st_chan[kPer], st_sp[kPer];
+      // ---- store: eight channels per round through the LDS stage ----
+      // Register e of a tile holds channel 16 * h + 4 * quad + e of the lane's voxel.  A round
+      // takes the registers e = 2p and 2p + 1 of the tiles of one h: every lane writes two
+      // channels, plane 2 * quad + (e & 1) of the stage holds channel
+      // 16 * h + 4 * quad + 2 * p + (e & 1).
+      int st_lds[kPer], st_slot[kPer], st_sp[kPer];
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
         const int item = tid + k * kColThreads;
         const int jj = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
         const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
-        st_lds[k] = jj * kPlane + row * kRowPad + f4 * 4;
-        st_chan[k] = (gx < dim && gy < dim && gz < dim) ? jj : -1;
+        st_lds[k] = jj * kPlaneS + row * kRowPad + f4 * 4;
+        st_slot[k] = (gx < dim && gy < dim && gz < dim) ? jj : -1;
         st_sp[k] = (gx * dim + gy) * dim + gz;
       }
-      auto store_round = [&](int r) {
-        const float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
+      auto store_round = [&](int h, int p) {
         lds_barrier();
-        float* ob = out_b + (size_t)(cbase + r * kStageCh) * chan_stride;
-        const int nch = min(kStageCh, nchan - r * kStageCh);
+        float* ob = out_b + (size_t)cbase * chan_stride;
 #pragma unroll
-        for (int k = 0; k < kPer; ++k) {
-          if (st_chan[k] >= 0 && st_chan[k] < nch) {
-            const v4f v = *reinterpret_cast<const v4f*>(stage + st_lds[k]);
-            float* dst = ob + (size_t)st_chan[k] * chan_stride + st_sp[k];
-            const int gz = z0 + ((tid + k * kColThreads) % 12) * 4;
-            if ((vec_store & 1) && gz + 3 < dim) {
-              // non-temporal: the grids are not read back soon, and the write-back of plain
-              // stores runs on into the next launch (binary occupancy: 0.65 ms against 0.85 ms)
-              __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(dst));
-            } else {
-              dst[0] = v.x;
-              if (gz + 1 < dim) dst[1] = v.y;
-              if (gz + 2 < dim) dst[2] = v.z;
-              if (gz + 3 < dim) dst[3] = v.w;
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+          for (int k = 0; k < kPer; ++k) {
+            const int slot = st_slot[k] + 4 * half;
+            const int ch = 16 * h + 4 * (slot >> 1) + 2 * p + (slot & 1);
+            if (st_slot[k] >= 0 && ch < nchan) {
+              const v4f v = *reinterpret_cast<const v4f*>(s_stage + st_lds[k] + 4 * half * kPlaneS);
+              float* dst = ob + (size_t)ch * chan_stride + st_sp[k];
+              const int gz = z0 + ((tid + k * kColThreads) % 12) * 4;
+              if ((vec_store & 1) && gz + 3 < dim) {
+                // non-temporal: the grids are not read back soon, and the write-back of plain
+                // stores runs on into the next launch (binary occupancy: 0.65 ms against 0.85 ms)
+                __builtin_nontemporal_store(v, reinterpret_cast<v4f*>(dst));
+              } else {
+                dst[0] = v.x;
+                if (gz + 1 < dim) dst[1] = v.y;
+                if (gz + 2 < dim) dst[2] = v.z;
+                if (gz + 3 < dim) dst[3] = v.w;
+              }
             }
           }
         }
       };
-      // Register e of a tile holds channel 16 * h + 4 * quad + e of the lane's voxel, so channels
-      // 4r .. 4r+3 are the four registers of the tiles with h = r / 4 in the lanes with
-      // quad == r % 4.
-      auto dump_round = [&](auto rc) {
-        constexpr int r = decltype(rc)::value;
-        if (quad == (r & 3)) {
-          float* stage = s_stage + (r & 1) * (kStageCh * kPlane);
+      auto dump_round = [&](auto hc, auto pc) {
+        constexpr int h = decltype(hc)::value, p = decltype(pc)::value;
+        lds_barrier();   // the stage (or the chunk's rows) has been read
 #pragma unroll
-          for (int blk = 0; blk < kBlocksPerWave; ++blk)
+        for (int blk = 0; blk < kBlocksPerWave; ++blk)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+          for (int t = 0; t < 4; ++t)
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                stage[e * kPlane + (t * 4 + jy) * kRowPad + (wave * kBlocksPerWave + blk) * 4 + jz] =
-                    sums[blk][t][r >> 2][e];
+            for (int ee = 0; ee < 2; ++ee)
+              s_stage[(2 * quad + ee) * kPlaneS + (t * 4 + jy) * kRowPad +
+                      (wave * kBlocksPerWave + blk) * 4 + jz] = sums[blk][t][h][2 * p + ee];
+      };
+      auto round = [&](auto hc, auto pc) {
+        constexpr int h = decltype(hc)::value, p = decltype(pc)::value;
+        if (nchan > 16 * h) {
+          dump_round(hc, pc);
+          store_round(h, p);
         }
       };
-      auto round = [&](auto rc) {
-        constexpr int r = decltype(rc)::value;
-        if (nchan > r * kStageCh) {
-          dump_round(rc);
-          store_round(r);
-        }
-      };
-      round(std::integral_constant<int, 0>{});
-      round(std::integral_constant<int, 1>{});
-      round(std::integral_constant<int, 2>{});
-      round(std::integral_constant<int, 3>{});
-      round(std::integral_constant<int, 4>{});
-      round(std::integral_constant<int, 5>{});
-      round(std::integral_constant<int, 6>{});
-      round(std::integral_constant<int, 7>{});
+      round(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+      round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+      round(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+      round(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
       lds_barrier();
     }
   }
@@ -385,14 +454,16 @@ hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, i
   const int vec_store = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0) &&
                          ((chan_stride * g.ntypes) % 4 == 0)) ? 1 : 0;
   const int groups = cols_per_side * ((cols_per_side + kColsPerGroup - 1) / kColsPerGroup);
+  // weight rows can be read four channels at a time
+  const int vec_weights = ((g.ntypes % 4 == 0) && ((reinterpret_cast<uintptr_t>(type_vector) & 15) == 0)) ? 1 : 0;
   if (binary)
     hipLaunchKernelGGL(splat_vector_mfma_kernel<true>, dim3(groups * slabs, nbatch),
                        dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
-                       out, cols_per_side, vec_store);
+                       out, cols_per_side, vec_store, vec_weights);
   else
     hipLaunchKernelGGL(splat_vector_mfma_kernel<false>, dim3(groups * slabs, nbatch),
                        dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
-                       out, cols_per_side, vec_store);
+                       out, cols_per_side, vec_store, vec_weights);
   return hipGetLastError();
 }
 
