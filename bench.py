@@ -86,6 +86,12 @@ def measured_traffic(kernel):
     return None
 
 
+def forward_traffic():
+    """Both launches of a forward call."""
+    parts = [measured_traffic("sort_atoms_kernel"), measured_traffic("splat_sorted_kernel")]
+    return None if None in parts else sum(parts)
+
+
 def cpu_baseline(cfg, ntypes, nsample, threads):
     """Oracle (CPU restatement of the reference loops) on the first nsample examples."""
     import oracle
@@ -329,8 +335,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round((fwd_gbs if dominant_fwd else bwd_gbs) / HBM_PEAK_GBS, 4),
-        "traffic": measured_traffic("splat_sorted_kernel" if dominant_fwd
-                                    else "backward_index_kernel"),
+        "traffic": forward_traffic() if dominant_fwd else measured_traffic("backward_index_kernel"),
         "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 counters of this command, not of this run)",
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
