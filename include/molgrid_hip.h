@@ -229,6 +229,13 @@ int mg_interpolate(float in_resolution, float in_dimension, float out_resolution
                    const float* out_centers, const float out_center_host[3], float* out,
                    void* stream);
 
+/* No counterpart in the reference: a switch for tests.  on != 0 makes every
+ * tile of the resampling kernel read its taps straight from global memory
+ * instead of staging them in LDS (otherwise only tiles that would overflow the
+ * staging buffers do); the values are the same bit for bit.  Process wide;
+ * returns the previous setting. */
+int mg_interpolate_force_gather(int on);
+
 /* Double precision arrays at the boundary.  The reference instantiates its GPU
  * overloads for Grid<double, N, true> outputs, gradients and coordinates too
  * (src/grid_maker.cu:293-294, 445-446, 460-466, 600; src/transform.cu:96;

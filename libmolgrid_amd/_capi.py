@@ -21,7 +21,7 @@ EXPORTED_SYMBOLS = (
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
     "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_vector", "mg_backward_index",
     "mg_backward_index_unrotated",
-    "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate",
+    "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate", "mg_interpolate_force_gather",
     "mg_narrow", "mg_widen",
 )
 
@@ -85,6 +85,7 @@ def _load():
                                    _vp, _f3, _vp, _f3, _vp, _vp]
     lib.mg_narrow.argtypes = [_vp, _vp, ctypes.c_size_t, _vp]
     lib.mg_widen.argtypes = [_vp, _vp, ctypes.c_size_t, _vp]
+    lib.mg_interpolate_force_gather.argtypes = [_i]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)
         if name not in ("mg_error_string", "mg_forward_index_workspace_size"):

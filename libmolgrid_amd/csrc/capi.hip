@@ -482,4 +482,6 @@ int mg_interpolate(float in_resolution, float in_dimension, float out_resolution
                                      (hipStream_t)stream));
 }
 
+int mg_interpolate_force_gather(int on) { return mg::set_interpolate_force_gather(on); }
+
 }  // extern "C"

@@ -9,8 +9,6 @@
 // loop does (src/grid_maker.cpp:226-270), so binary mode (`+= weight`) is
 // reproduced bit for bit.  The tile is staged through LDS and streamed out as
 // float4 rows.
-#include <cstdlib>
-
 #include "kernels.h"
 #include "splat_common.h"
 

@@ -22,7 +22,7 @@
 //
 // The coordinate chain keeps the reference's rounding order; taps outside the input grid read as
 // zero and integral coordinates get weight zero (src/grid_interpolater.cu:17-58).
-#include <cstdlib>
+#include <atomic>
 
 #include "kernels.h"
 
@@ -433,7 +433,11 @@ __global__ __launch_bounds__(kThreads) void interpolate_gather_kernel(
   }
 }
 
+std::atomic<int> g_force_gather{0};
+
 }  // namespace
+
+int set_interpolate_force_gather(int on) { return g_force_gather.exchange(on != 0 ? 1 : 0); }
 
 hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_centers,
                               const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
@@ -448,8 +452,7 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
     const int tiles = tiles_x * tiles_x * tiles_z;
     const int groups = (nbatch + 7) / 8;
     // test hook: every tile takes the gather path (otherwise only a safety net)
-    const char* hook = getenv("MOLGRID_HIP_INTERP_PLAIN_STAGING");
-    const int gather_only = (hook != nullptr && hook[0] == '1') ? 1 : 0;
+    const int gather_only = g_force_gather.load();
     hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), 0,
                        stream, p, nbatch, tiles_x, tiles_z, in_centers, in, quats, rot_centers,
                        translations, out_centers, out, gather_only);

@@ -82,6 +82,10 @@ hipError_t launch_backward_gradients(const GridArg& g, const BatchArg& batch, in
                                      float* diffdiff, float* atom_diffdiff, float* type_diffdiff,
                                      bool radii_type_indexed, hipStream_t stream);
 
+// Test hook: 1 makes every tile of the tiled resampling kernel gather its taps from global memory
+// (normally a safety net); returns the previous setting.
+int set_interpolate_force_gather(int on);
+
 hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_centers,
                               const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
                               const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,

@@ -69,7 +69,7 @@ def test_batch_config4_shape_vs_oracle(mg):
     assert_close(out.cpu().numpy(), ref, what="config 4")
 
 
-def test_plain_staging_path_gives_the_same_values(mg, monkeypatch):
+def test_plain_staging_path_gives_the_same_values(mg):
     """The kernel's safety net (whole-window staging, taken when a tile would need more input voxels
     than the pipelined path holds) is not reachable with valid resolutions; the library's test hook
     forces it, and it must reproduce the pipelined path bit for bit."""
@@ -82,11 +82,14 @@ def test_plain_staging_path_gives_the_same_values(mg, monkeypatch):
     gi = mg.GridInterpolater(0.5, 23.5, 0.5, 23.5)
     fast = torch.empty((B, K, D, D, D), device="cuda")
     gi.forward_batch(src, quats, zeros, trans, fast)
-    monkeypatch.setenv("MOLGRID_HIP_INTERP_PLAIN_STAGING", "1")
-    plain = torch.full((B, K, D, D, D), 7.0, device="cuda")
-    gi.forward_batch(src, quats, zeros, trans, plain)
-    torch.cuda.synchronize()
-    monkeypatch.delenv("MOLGRID_HIP_INTERP_PLAIN_STAGING")
+    from libmolgrid_amd import _capi
+    assert _capi.lib.mg_interpolate_force_gather(1) == 0
+    try:
+        plain = torch.full((B, K, D, D, D), 7.0, device="cuda")
+        gi.forward_batch(src, quats, zeros, trans, plain)
+        torch.cuda.synchronize()
+    finally:
+        assert _capi.lib.mg_interpolate_force_gather(0) == 1
     assert torch.equal(fast, plain)
 
 
