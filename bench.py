@@ -205,6 +205,16 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
             ms, nbytes, grids_per_s=round(16 / (ms * 1e-3), 1),
             workload="configs[3]: 16 x 10,000 atoms, 28x96^3 at 0.25 A")
         del out
+    # the same atoms with radii by type instead of by atom (a density per atom AND channel: no
+    # matrix product, 28 times the density evaluations)
+    gv = mg.GridMaker(0.25, 23.75, False, True)
+    tr = torch.as_tensor(np.random.default_rng(11).uniform(1.2, 2.0, (16, 28)).astype(np.float32)).cuda()
+    out = torch.empty((16,) + gv.grid_dimensions(28), device="cuda")
+    ms = event_ms(lambda: gv.forward_batch(ab, vcen, vc, vt, tr, out), 3, warmup=1)
+    res["forward_vector_type_radii"] = entry(
+        ms, out.numel() * 4 + vc.shape[0] * (12 + 4 * 28), grids_per_s=round(16 / (ms * 1e-3), 1),
+        workload="configs[3] atoms with type-indexed radii (16 x 28 radii), Gaussian")
+    del out
     return res
 
 
