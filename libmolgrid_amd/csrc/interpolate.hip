@@ -8,7 +8,7 @@
 // bounding box is never touched; a bit per position, one word per (x, y) row), numbers the marked
 // positions that lie inside the input grid in window order, and deals them out evenly to its
 // threads.  Per channel the threads stage those positions -- and nothing else -- into an LDS
-// buffer in that order (12 KB instead of the 39 KB of the whole window, so that four workgroups
+// buffer in that order (12 KB instead of the 39 KB of the whole window, so that three workgroups
 // share a CU), and every thread reads its eight taps from the slots it looked up once; a tap
 // outside the input grid reads a cell that holds zero.  The source position, the tap slots and
 // the weights are computed once per output voxel and reused for every channel.  Staging runs two
