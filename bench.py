@@ -397,6 +397,23 @@ def main():
             "backward_atom_grads_per_s": round(passes * r1["atoms"] / r1["backward_s"], 1),
         }
         try:
+            # resampling (configuration 4) on the CPU: a few grids, single thread
+            import oracle
+            import synth as _synth
+            nint = 16
+            rng = np.random.default_rng(4)
+            src = rng.standard_normal((nint, T, D, D, D)).astype(np.float32)
+            zeros = np.zeros((nint, 3), np.float32)
+            t0 = time.perf_counter()
+            oracle.interpolate_batch(0.5, 23.5, 0.5, 23.5, zeros, src,
+                                     _synth.random_quaternions(rng, nint), zeros,
+                                     rng.uniform(-1.5, 1.5, (nint, 3)).astype(np.float32), zeros,
+                                     nthreads=1)
+            cpu["interpolated_grids_per_s"] = round(nint / (time.perf_counter() - t0), 2)
+            del src
+        except Exception as e:  # pragma: no cover
+            cpu["interpolated_grids_per_s"] = {"error": str(e)}
+        try:
             import oracle
             nt = min(oracle.max_threads(), 16)
             if nt > 1:
