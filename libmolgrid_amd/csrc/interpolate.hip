@@ -6,11 +6,12 @@
 // input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), marks the
 // window positions that some tap of the tile reads (about 40 % of the window: the rest of the
 // bounding box is never touched; a bit per position, one word per (x, y) row), numbers the marked
-// positions that lie inside the input grid in window order, and deals them out evenly to its
-// threads.  Per channel the threads stage those positions -- and nothing else -- into an LDS
-// buffer in that order (12 KB instead of the 39 KB of the whole window, so that three workgroups
-// share a CU), and every thread reads its eight taps from the slots it looked up once; a tap
-// outside the input grid reads a cell that holds zero.  The source position, the tap slots and
+// positions in window order, and deals them out evenly to its threads.  Per channel the threads
+// stage those positions -- and nothing else -- into an LDS buffer in that order (12 KB instead
+// of the 39 KB of the whole window, so that three workgroups share a CU); a position outside the
+// input grid is staged as zero (its load lies past the end of the buffer descriptor, which
+// returns zero).  Every thread reads its eight taps from the slots it looked up once, the two of
+// a row, which are neighbours, with one LDS instruction.  The source position, the tap slots and
 // the weights are computed once per output voxel and reused for every channel.  Staging runs two
 // channels ahead of the interpolation: two register sets and two LDS buffers, one barrier per
 // channel.  Workgroups are numbered so that all tiles of one example run on the same XCD (they
@@ -67,6 +68,8 @@ __device__ __forceinline__ float lerp3(float p000, float p001, float p010, float
 }
 
 // ---------------------------------------------------------------------------------------------
+struct alignas(4) TapPair { float lo, hi; };   // the taps at z and z + 1: neighbours in a buffer
+
 constexpr int kTileX = 8, kTileY = 8, kTileZ = 16;   // output tile; 16 voxels of z = one 64-byte line
 constexpr int kTileThreads = 512;              // two output voxels (x and x + 4) per thread
 constexpr int kTileWaves = kTileThreads / 64;
@@ -76,7 +79,7 @@ constexpr int kRows = kWin * kWin;             // (x, y) rows of the window
 constexpr int kRowsPad = 448;
 constexpr int kFewRounds = 6;                  // staged elements per thread and channel
 constexpr int kSlots = kFewRounds * kTileThreads;   // 3,072 >= the 2,800 input voxels a tile can need
-constexpr int kBuf = kSlots + 4;               // floats per buffer: the slots and a cell that holds zero
+constexpr int kBuf = kSlots + 4;               // floats per buffer
 // longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
 constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
 
@@ -191,15 +194,17 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   // order (row by row, z ascending): slot n of a buffer holds the n-th of them, and thread t stages
   // slots t, t + 512, ...  One thread per row counts the row's positions, a prefix sum over the
   // workgroup gives the row its first slot.
-  unsigned zmask = 0;
+  unsigned zmask = 0, zinside = 0;   // positions in use; those of them inside the input grid
   int row_src = 0;
   if (tid < kRows) {
     const int ex = tid / kWin, ey = tid - ex * kWin;
     const int gx = wlo[0] + ex, gy = wlo[1] + ey;
     row_src = (gx * id + gy) * id + wlo[2];
-    if (ex < wn[0] && ey < wn[1] && gx >= 0 && gx < id && gy >= 0 && gy < id) {
+    if (ex < wn[0] && ey < wn[1]) {
+      zmask = s_rowmask[tid];
       const int zl = max(0, -wlo[2]), zh = min(wn[2], id - wlo[2]);   // z positions inside the grid
-      if (zh > zl) zmask = s_rowmask[tid] & ((1u << zh) - 1u) & ~((1u << zl) - 1u);
+      if (gx >= 0 && gx < id && gy >= 0 && gy < id && zh > zl)
+        zinside = zmask & ((1u << zh) - 1u) & ~((1u << zl) - 1u);
     }
   }
   const int mine = __popc(zmask);
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
       while (m != 0) {
         const int ez = __builtin_ctz(m);
         m &= m - 1u;
-        s_list[slot++] = row_src + ez;
+        s_list[slot++] = ((zinside >> ez) & 1u) ? row_src + ez : -1;   // -1: outside, stays zero
       }
     }
   }
@@ -275,7 +280,9 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   // ---- slots of this thread's taps (byte offsets inside a buffer; the zero cell for a tap that
   // lies outside the input grid), and the sources of the slots it stages
-  unsigned tap_off[kVox][4];   // two 16-bit byte offsets each: the taps at z and z + 1
+  // The taps at z and z + 1 of a row are both in use (this voxel marked them), so they sit in
+  // consecutive slots: one byte offset per (x, y) row of the voxel, two 16-bit offsets a register.
+  unsigned tap_off[kVox][2];
 #pragma unroll
   for (int v = 0; v < kVox; ++v) {
     const int r0 = wpos[v] >> 8, wz = wpos[v] & 255;
@@ -283,26 +290,24 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
     for (int q = 0; q < 4; ++q) {
       const int r = r0 + (q >> 1) * kWin + (q & 1);
       const unsigned m = s_rowmask[r];
-      const int first = s_rowstart[r];
-      unsigned both = 0;
-#pragma unroll
-      for (int dz = 0; dz < 2; ++dz) {
-        const int bit = wz + dz;
-        const bool have = (m >> bit) & 1u;
-        const int slot = first + __popc(m & ((1u << bit) - 1u));
-        both |= ((unsigned)(have ? slot : kSlots) * 4u) << (16 * dz);
-      }
-      tap_off[v][q] = both;
+      const int slot = s_rowstart[r] + __popc(m & ((1u << wz) - 1u));
+      // (a voxel outside the output grid marked nothing: its offsets stay inside the buffer and
+      // its values are dropped)
+      const unsigned off = (unsigned)min(slot, kSlots - 2) * 4u;
+      if (q & 1) tap_off[v][q >> 1] |= off << 16;
+      else tap_off[v][q >> 1] = off;
     }
   }
   int st_src[kFewRounds];   // byte offset inside one input channel
 #pragma unroll
   for (int e = 0; e < kFewRounds; ++e) {
     const int slot = tid + e * kTileThreads;
-    st_src[e] = (slot < planned ? s_list[slot] : 0) * 4;   // a slot past the plan is read by no tap
+    // a position outside the input grid, or a slot past the plan, is an offset past the end of the
+    // descriptor below: the load returns zero without touching memory
+    const int src_elem = slot < planned ? s_list[slot] : -1;
+    st_src[e] = src_elem >= 0 ? src_elem * 4 : 0x7ffffff0;
   }
   __syncthreads();   // the tables have been read: the buffers can be filled
-  if (tid == 0) s_buf[kSlots] = s_buf[kBuf + kSlots] = 0.f;
 
   // Two register sets, so that the loads of a channel are issued a whole channel before they are
   // needed: while channel ch is interpolated from one buffer, channel ch + 1 is written to the
@@ -345,8 +350,10 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
       float t8[8];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        t8[2 * q] = *reinterpret_cast<const float*>(buf + (tap_off[v][q] & 0xffffu));
-        t8[2 * q + 1] = *reinterpret_cast<const float*>(buf + (tap_off[v][q] >> 16));
+        const unsigned off = (q & 1) ? tap_off[v][q >> 1] >> 16 : tap_off[v][q >> 1] & 0xffffu;
+        const TapPair pair = *reinterpret_cast<const TapPair*>(buf + off);   // one ds_read2_b32
+        t8[2 * q] = pair.lo;
+        t8[2 * q + 1] = pair.hi;
       }
       const float val = lerp3(t8[0], t8[1], t8[2], t8[3], t8[4], t8[5], t8[6], t8[7], frac[v][0],
                               frac[v][1], frac[v][2]);
