@@ -328,6 +328,14 @@ def main():
     ms_tr = event_ms(k_transform, it)
     in_step = step_breakdown([k_transform, k_forward, k_backward, k_unrotate], it)
     ms_bwd_unrot = event_ms(k_backward_unrotated, it)
+    # What the write stream alone costs on this box: the same forward call with every atom's type
+    # set to "ignored" (the sort launch does its work and drops them, the splat launch stores
+    # zeros in its usual pattern and order, with no arithmetic), and a plain fill of the tensor.
+    types_none = torch.full_like(types, -1.0)
+    ms_fwd_stores = event_ms(lambda: gm.forward_batch(offsets, centers, moved, types_none, radii, grid), it)
+    ms_fill = event_ms(lambda: grid.zero_(), it)
+    del types_none
+    k_forward()                                   # the grids of the step again
 
     grid_bytes = B * T * D ** 3 * 4
     fwd_bytes = grid_bytes + n_atoms * 20          # grid written once + coords/type/radius read
@@ -349,6 +357,12 @@ def main():
         "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 counters of this command, not of this run)",
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
+        # measured in this run: the forward call with its arithmetic removed, and a plain fill
+        "write_stream_alone": {
+            "forward_call_all_atoms_ignored_ms": round(ms_fwd_stores, 4),
+            "frac": round(fwd_bytes / (ms_fwd_stores * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "torch_fill_ms": round(ms_fill, 4),
+            "torch_fill_frac": round(grid_bytes / (ms_fill * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         # the same kernel between the other launches of the step (see step_breakdown)
         "in_step_ms": round(in_step[1] if dominant_fwd else in_step[2], 4),
         "in_step_frac": round((fwd_bytes / in_step[1] if dominant_fwd else bwd_bytes / in_step[2])
