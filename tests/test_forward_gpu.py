@@ -57,6 +57,7 @@ def test_density_profile_closed_form(mg):
     (0.5, 23.5, 28, 300),   # dim 48
     (0.5, 29.5, 4, 500),    # dim 60: two slabs in z, the second one partial
     (0.25, 25.25, 3, 400),  # dim 102: three slabs, rows that are not a multiple of four voxels
+    (0.5, 31.5, 4, 400),    # dim 64: two slabs of 32 voxels (whole cache lines) instead of 48 + 16
 ])
 @pytest.mark.parametrize("binary", [False, True])
 def test_small_random_vs_oracle(mg, res, dimension, ntypes, natoms, binary):
