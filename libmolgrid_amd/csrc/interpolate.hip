@@ -1,14 +1,15 @@
 // Trilinear resampling of a batch of 4-D grids through an inverse rigid transform
 // (GridInterpolater::forward, src/grid_interpolater.cpp:16-48).
 //
-// Main kernel (interpolate_tiled_kernel): one workgroup owns an 8x8x16 tile of output voxels (16
-// along z, so that its stores are whole 64-byte lines).  The tile maps to a rotated box in the
-// input grid; the workgroup finds that box's bounding window (at most 21^3 voxels), marks the
-// window positions that some tap of the tile reads (about 40 % of the window: the rest of the
+// Main kernel (interpolate_tiled_kernel): one workgroup owns an 8x16x16 tile of output voxels (16
+// along z, so that its stores are 64-byte pieces; four voxels per thread).  The tile maps to a
+// rotated box in the input grid; the workgroup finds that box's bounding window (at most 26^3
+// voxels), marks the window positions that some tap of the tile reads (a sixth of the window: the rest of the
 // bounding box is never touched; a bit per position, one word per (x, y) row), numbers the marked
 // positions in window order, and deals them out evenly to its threads.  Per channel the threads
 // stage those positions -- and nothing else -- into an LDS buffer in that order (12 KB instead
-// of the 39 KB of the whole window, so that three workgroups share a CU); a position outside the
+// of the 70 KB of the whole window; about 2,850 values for the 2,048 voxels of a tile, 1.4 each,
+// where an 8x8x16 tile needs 1.5 each); a position outside the
 // input grid is staged as zero (its load lies past the end of the buffer descriptor, which
 // returns zero).  Every thread reads its eight taps from the slots it looked up once, the two of
 // a row, which are neighbours, with one LDS instruction.  The source position, the tap slots and
@@ -70,21 +71,23 @@ __device__ __forceinline__ float lerp3(float p000, float p001, float p010, float
 // ---------------------------------------------------------------------------------------------
 struct alignas(4) TapPair { float lo, hi; };   // the taps at z and z + 1: neighbours in a buffer
 
-constexpr int kTileX = 8, kTileY = 8, kTileZ = 16;   // output tile; 16 voxels of z = one 64-byte line
-constexpr int kTileThreads = 512;              // two output voxels (x and x + 4) per thread
+constexpr int kTileX = 8, kTileY = 16, kTileZ = 16;  // output tile; 16 voxels of z = one 64-byte line
+constexpr int kTileThreads = 512;              // four output voxels (x, x + 2, x + 4, x + 6) per thread
 constexpr int kTileWaves = kTileThreads / 64;
 constexpr int kVox = kTileX * kTileY * kTileZ / kTileThreads;
-constexpr int kWin = 21;                       // largest window side (the tile's bounding box in the input)
+constexpr int kWin = 26;                       // largest window side (the tile's bounding box in the input)
 constexpr int kRows = kWin * kWin;             // (x, y) rows of the window
-constexpr int kRowsPad = 448;
-constexpr int kFewRounds = 6;                  // staged elements per thread and channel
-constexpr int kSlots = kFewRounds * kTileThreads;   // 3,072 >= the 2,800 input voxels a tile can need
+constexpr int kRowsPad = 704;
+constexpr int kRowsPer = (kRows + kTileThreads - 1) / kTileThreads;   // window rows a thread plans: 2
+constexpr int kFewRounds = 6;                   // staged elements per thread and channel
+constexpr int kSlots = kFewRounds * kTileThreads;   // 3,072: a tile needs 2,830 input voxels on average, 2,940 at
+                                               // most over random rotations (more: the gather path below)
 constexpr int kBuf = kSlots + 4;               // floats per buffer
 // longest image of the tile's diagonal, in units of (out_res / in_res) input voxels
-constexpr float kTileDiagonal = 17.972f;       // sqrt(7^2 + 7^2 + 15^2)
+constexpr float kTileDiagonal = 22.339f;       // sqrt(7^2 + 15^2 + 15^2)
 
 __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
-    InterpArg p, int nbatch, int tiles_x, int tiles_z, Vec3Arg in_centers,
+    InterpArg p, int nbatch, int tiles_x, int tiles_y, int tiles_z, Vec3Arg in_centers,
     const float* __restrict__ in, Vec4Arg quats, Vec3Arg rot_centers, Vec3Arg translations,
     Vec3Arg out_centers, float* __restrict__ out, int gather_only) {
   // Two buffers of staged input values, in plan order (below).  While the plan is made the same
@@ -101,19 +104,20 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   // workgroup -> (example, tile): consecutive workgroups are dealt round-robin to the 8 XCDs, so
   // example b is pinned to XCD b % 8 and its tiles run there in z-fastest order
-  const int tiles = tiles_x * tiles_x * tiles_z;
+  const int tiles = tiles_x * tiles_y * tiles_z;
   const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
   const int b = (slot_id / tiles) * 8 + xcd;
   if (b >= nbatch) return;
   const int tile = slot_id % tiles;
-  const int tz = tile % tiles_z, ty = (tile / tiles_z) % tiles_x;
-  const int tx = tile / (tiles_z * tiles_x);
+  const int tz = tile % tiles_z, ty = (tile / tiles_z) % tiles_y;
+  const int tx = tile / (tiles_z * tiles_y);
 
   const int od = p.out_dim, id = p.in_dim;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   // 16 consecutive lanes run along z: one store instruction writes whole 64-byte lines
-  const int i0 = tx * kTileX + (tid >> 7), j = ty * kTileY + ((tid >> 4) & 7), k = tz * kTileZ + (tid & 15);
+  static_assert(kTileZ == 16 && kTileY == 16 && kTileX * kTileY * kTileZ == kVox * kTileThreads, "thread to voxel map");
+  const int i0 = tx * kTileX + (tid >> 8), j = ty * kTileY + ((tid >> 4) & 15), k = tz * kTileZ + (tid & 15);
 
   const float3 ic = load3(in_centers, b), oc = load3(out_centers, b);
   const float3 c = load3(rot_centers, b), t = load3(translations, b);
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   const float4 qinvinv = quat_inverse(qinv);
 
   // ---- window of the tile: bounding box of the images of its eight corners -----------------
-  if (tid < kRowsPad) s_rowmask[tid] = 0u;
+  for (int r = tid; r < kRowsPad; r += kTileThreads) s_rowmask[r] = 0u;
   if (tid < 8) {
     const int ci = min(tx * kTileX + ((tid >> 2) & 1) * (kTileX - 1), od - 1);
     const int cj = min(ty * kTileY + ((tid >> 1) & 1) * (kTileY - 1), od - 1);
@@ -194,20 +198,28 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   // order (row by row, z ascending): slot n of a buffer holds the n-th of them, and thread t stages
   // slots t, t + 512, ...  One thread per row counts the row's positions, a prefix sum over the
   // workgroup gives the row its first slot.
-  unsigned zmask = 0, zinside = 0;   // positions in use; those of them inside the input grid
-  int row_src = 0;
-  if (tid < kRows) {
-    const int ex = tid / kWin, ey = tid - ex * kWin;
-    const int gx = wlo[0] + ex, gy = wlo[1] + ey;
-    row_src = (gx * id + gy) * id + wlo[2];
-    if (ex < wn[0] && ey < wn[1]) {
-      zmask = s_rowmask[tid];
-      const int zl = max(0, -wlo[2]), zh = min(wn[2], id - wlo[2]);   // z positions inside the grid
-      if (gx >= 0 && gx < id && gy >= 0 && gy < id && zh > zl)
-        zinside = zmask & ((1u << zh) - 1u) & ~((1u << zl) - 1u);
+  // (a thread plans the window rows tid, tid + 512, ...: their slots follow each other)
+  unsigned zmask[kRowsPer], zinside[kRowsPer];   // positions in use; those inside the input grid
+  int row_src[kRowsPer];
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < kRowsPer; ++u) {
+    const int row = tid + u * kTileThreads;
+    zmask[u] = zinside[u] = 0;
+    row_src[u] = 0;
+    if (row < kRows) {
+      const int ex = row / kWin, ey = row - ex * kWin;
+      const int gx = wlo[0] + ex, gy = wlo[1] + ey;
+      row_src[u] = (gx * id + gy) * id + wlo[2];
+      if (ex < wn[0] && ey < wn[1]) {
+        zmask[u] = s_rowmask[row];
+        const int zl = max(0, -wlo[2]), zh = min(wn[2], id - wlo[2]);   // z positions inside the grid
+        if (gx >= 0 && gx < id && gy >= 0 && gy < id && zh > zl)
+          zinside[u] = zmask[u] & ((1u << zh) - 1u) & ~((1u << zl) - 1u);
+      }
     }
+    mine += __popc(zmask[u]);
   }
-  const int mine = __popc(zmask);
   int incl = mine;                                         // inclusive scan over the wave
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
@@ -227,17 +239,22 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
   // (the buffer loads of the main path address one example's input with 32 bits)
   const bool gather = rounds_used > kFewRounds || gather_only ||
                       (size_t)p.channels * id * id * id * sizeof(float) >= 0x7fffffffull;
-  if (tid < kRows) {
-    s_rowmask[tid] = zmask;
-    s_rowstart[tid] = slot0;
-    if (!gather) {
-      unsigned m = zmask;
-      int slot = slot0;
-      while (m != 0) {
-        const int ez = __builtin_ctz(m);
-        m &= m - 1u;
-        s_list[slot++] = ((zinside >> ez) & 1u) ? row_src + ez : -1;   // -1: outside, stays zero
+#pragma unroll
+  for (int u = 0; u < kRowsPer; ++u) {
+    const int row = tid + u * kTileThreads;
+    if (row < kRows) {
+      s_rowmask[row] = zmask[u];
+      s_rowstart[row] = slot0;
+      unsigned m = zmask[u];
+      if (!gather) {
+        int slot = slot0;
+        while (m != 0) {
+          const int ez = __builtin_ctz(m);
+          m &= m - 1u;
+          s_list[slot++] = ((zinside[u] >> ez) & 1u) ? row_src[u] + ez : -1;   // -1: outside, stays zero
+        }
       }
+      slot0 += __popc(zmask[u]);
     }
   }
   __syncthreads();
@@ -250,7 +267,7 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   if (gather) {
     // More positions than the buffers hold.  The launcher sends only resolution ratios here for
-    // which a tile needs at most 2,800 input voxels, so this is a safety net (and a test hook):
+    // which a tile needs fewer input voxels than the buffers hold, so this is a safety net (and a test hook):
     // every thread gathers its taps from global memory, with the weights and the order of the
     // sums of the main path.
     float* dst = out + (size_t)b * C * out_points + ((size_t)i0 * od + j) * od + k;
@@ -450,18 +467,19 @@ hipError_t launch_interpolate(const InterpArg& p, int nbatch, const Vec3Arg& in_
                               const float* in, const Vec4Arg& quats, const Vec3Arg& rot_centers,
                               const Vec3Arg& translations, const Vec3Arg& out_centers, float* out,
                               hipStream_t stream) {
-  // The image of an 8 x 8 x 16 output tile spans at most kTileDiagonal * (out_res / in_res) input
+  // The image of an 8 x 16 x 16 output tile spans at most kTileDiagonal * (out_res / in_res) input
   // voxels along an axis; with the two extra taps and the rounding slack it must fit the window.
   const float span = kTileDiagonal * (p.out_resolution / p.in_resolution);
   if (span + 3.0f <= (float)kWin) {
     const int tiles_x = (p.out_dim + kTileX - 1) / kTileX;
+    const int tiles_y = (p.out_dim + kTileY - 1) / kTileY;
     const int tiles_z = (p.out_dim + kTileZ - 1) / kTileZ;
-    const int tiles = tiles_x * tiles_x * tiles_z;
+    const int tiles = tiles_x * tiles_y * tiles_z;
     const int groups = (nbatch + 7) / 8;
     // test hook: every tile takes the gather path (otherwise only a safety net)
     const int gather_only = g_force_gather.load();
     hipLaunchKernelGGL(interpolate_tiled_kernel, dim3(groups * tiles * 8), dim3(kTileThreads), 0,
-                       stream, p, nbatch, tiles_x, tiles_z, in_centers, in, quats, rot_centers,
+                       stream, p, nbatch, tiles_x, tiles_y, tiles_z, in_centers, in, quats, rot_centers,
                        translations, out_centers, out, gather_only);
     return hipGetLastError();
   }
