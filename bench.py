@@ -8,6 +8,7 @@ N(0,1) upstream gradient and the un-rotation of those gradients.  All inputs are
 resident in HBM before the timed region.  One JSON line is printed.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+                    [--no-write-stream] [--graph]
 """
 import argparse
 import json
@@ -228,6 +229,10 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the other workloads (sparse upstream gradient, vector types at "
                          "28x96^3, resampling), which are measured after the timed steps")
+    ap.add_argument("--no-write-stream", action="store_true",
+                    help="skip the forward call with every atom ignored (the write stream alone) "
+                         "and the plain fill: for profiling runs, whose per-kernel means then "
+                         "cover the real calls only")
     ap.add_argument("--graph", action="store_true",
                     help="replay the four launches of a step as one captured HIP graph (measured: "
                          "no faster than launching them one by one, which is the default)")
@@ -317,9 +322,11 @@ def main():
     t0 = time.perf_counter()
     for _ in range(args.steps):
         run_step()
+    t_enqueued = time.perf_counter()              # the host has handed over every launch
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
+    enqueue_ms_per_step = (t_enqueued - t0) / args.steps * 1e3
 
     # per-kernel durations (events on the launch stream)
     it = max(args.steps, 10)
@@ -331,11 +338,13 @@ def main():
     # What the write stream alone costs on this box: the same forward call with every atom's type
     # set to "ignored" (the sort launch does its work and drops them, the splat launch stores
     # zeros in its usual pattern and order, with no arithmetic), and a plain fill of the tensor.
-    types_none = torch.full_like(types, -1.0)
-    ms_fwd_stores = event_ms(lambda: gm.forward_batch(offsets, centers, moved, types_none, radii, grid), it)
-    ms_fill = event_ms(lambda: grid.zero_(), it)
-    del types_none
-    k_forward()                                   # the grids of the step again
+    ms_fwd_stores = ms_fill = None
+    if not args.no_write_stream:
+        types_none = torch.full_like(types, -1.0)
+        ms_fwd_stores = event_ms(lambda: gm.forward_batch(offsets, centers, moved, types_none, radii, grid), it)
+        ms_fill = event_ms(lambda: grid.zero_(), it)
+        del types_none
+        k_forward()                               # the grids of the step again
 
     grid_bytes = B * T * D ** 3 * 4
     fwd_bytes = grid_bytes + n_atoms * 20          # grid written once + coords/type/radius read
@@ -358,7 +367,7 @@ def main():
         "algorithmic_bytes_per_launch": fwd_bytes if dominant_fwd else bwd_bytes,
         "avg_launch_ms": round(ms_fwd if dominant_fwd else ms_bwd, 4),
         # measured in this run: the forward call with its arithmetic removed, and a plain fill
-        "write_stream_alone": {
+        "write_stream_alone": None if ms_fwd_stores is None else {
             "forward_call_all_atoms_ignored_ms": round(ms_fwd_stores, 4),
             "frac": round(fwd_bytes / (ms_fwd_stores * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "torch_fill_ms": round(ms_fill, 4),
@@ -447,6 +456,9 @@ def main():
         "warmup": args.warmup,
         "launch": "hip graph replay" if args.graph else "eager",
         "ms_per_step": round(ms_per_step, 4),
+        # wall time the host needs to enqueue a step (the timed loop before its synchronize): when
+        # this comes close to ms_per_step the loop is bound by the host, not by the kernels
+        "enqueue_ms_per_step": round(enqueue_ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -1,7 +1,8 @@
 // C ABI of the gridding library: argument checks, then the kernel launches of the call on the
 // caller's stream.  Nothing here synchronises; the only allocation is the workspace that
-// mg_forward_index keeps per device (mg_forward_index_ws takes the caller's instead).
+// mg_forward_index keeps per device and stream (mg_forward_index_ws takes the caller's instead).
 #include <cmath>
+#include <cstdint>
 #include <cstring>
 #include <mutex>
 
@@ -173,6 +174,8 @@ int check_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
     return MG_OK;
   }
   if (out == nullptr) return MG_ERR_NULL_POINTER;
+  // atoms_per_example == 0 means "no atoms at all" (whatever the offsets say: the kernels are then
+  // given an empty batch and never touch the arrays, which may be missing)
   const bool has_atoms = atoms_per_example > 0;
   if (has_atoms && (coords == nullptr || type_index == nullptr || radii == nullptr))
     return MG_ERR_NULL_POINTER;
@@ -184,7 +187,8 @@ int forward_index_with(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
                        const float grid_center_host[3], const float* coords,
                        const float* type_index, const float* radii, int ntypes, float* out,
                        void* workspace, size_t workspace_bytes, void* stream) {
-  BatchArg batch{atom_offsets, atoms_per_example};
+  // no slot for any atom: every example is empty, the offsets are not looked at
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   const hipError_t e = launch_forward_sorted(
       grid_arg(g, ntypes), batch, nbatch, vec3(grid_centers, grid_center_host), coords, type_index,
       radii, out, g->binary != 0, needs_exact(g), workspace, workspace_bytes, (hipStream_t)stream);
@@ -192,13 +196,20 @@ int forward_index_with(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
   return from_hip(e);
 }
 
-// Workspace of mg_forward_index, one per device, grown when a call needs more.
-struct DeviceWorkspace {
+// Workspaces of mg_forward_index: one per (device, stream), grown when a call needs more.  A
+// block that became too small is kept until the process ends (launches already enqueued may still
+// use it, and a free would wait for the device); blocks grow by half at least, so what is kept
+// is bounded by twice the largest.
+struct StreamWorkspace {
+  int device = -1;
+  void* stream = nullptr;
   void* ptr = nullptr;
   size_t bytes = 0;
 };
 constexpr int kMaxDevices = 64;
-DeviceWorkspace g_workspace[kMaxDevices];
+constexpr int kMaxWorkspaces = 256;
+StreamWorkspace g_workspace[kMaxWorkspaces];
+int g_workspaces = 0;
 std::mutex g_workspace_mutex;
 
 }  // namespace
@@ -219,6 +230,7 @@ int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
                                     radii, ntypes, out, &nothing);
   if (s != MG_OK || nothing) return s;
   if (workspace == nullptr) return MG_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return MG_ERR_INVALID_ARGUMENT;
   if (workspace_bytes < mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes))
     return MG_ERR_INVALID_ARGUMENT;
   return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
@@ -239,28 +251,30 @@ int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offs
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return from_hip(e);
-  if (dev < 0 || dev >= kMaxDevices) return MG_ERR_UNSUPPORTED;
-  void* workspace = nullptr;
-  size_t bytes = 0;
-  {
-    std::lock_guard<std::mutex> lock(g_workspace_mutex);
-    DeviceWorkspace& w = g_workspace[dev];
-    if (w.bytes < need) {
-      // hipFree waits for the device, so no launch is still using the old block
-      if (w.ptr != nullptr) (void)hipFree(w.ptr);
-      w.ptr = nullptr;
-      w.bytes = 0;
-      const size_t want = need + need / 2;
-      e = hipMalloc(&w.ptr, want);
-      if (e != hipSuccess) return from_hip(e);
-      w.bytes = want;
-    }
-    workspace = w.ptr;
-    bytes = w.bytes;
+  // The lock is held until both launches are enqueued: calls of several host threads on one
+  // stream then follow each other in the stream and may share its block; calls on different
+  // streams get different blocks.
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  StreamWorkspace* w = nullptr;
+  for (int i = 0; i < g_workspaces; ++i)
+    if (g_workspace[i].device == dev && g_workspace[i].stream == stream) w = &g_workspace[i];
+  if (w == nullptr) {
+    if (g_workspaces == kMaxWorkspaces) return MG_ERR_UNSUPPORTED;   // use mg_forward_index_ws
+    w = &g_workspace[g_workspaces++];
+    w->device = dev;
+    w->stream = stream;
+  }
+  if (w->bytes < need) {
+    void* block = nullptr;
+    const size_t want = need + need / 2;
+    e = hipMalloc(&block, want);
+    if (e != hipSuccess) return from_hip(e);
+    w->ptr = block;                    // the block before it stays allocated
+    w->bytes = want;
   }
   return forward_index_with(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
-                            grid_center_host, coords, type_index, radii, ntypes, out, workspace, bytes,
-                            stream);
+                            grid_center_host, coords, type_index, radii, ntypes, out, w->ptr,
+                            w->bytes, stream);
 }
 
 namespace {

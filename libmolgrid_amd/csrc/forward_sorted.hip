@@ -141,16 +141,22 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
   const int wb = begin + wave * per, we = min(end, wb + per);
   const bool cached = per <= kCached * kWave;
 
-  // key of an atom among this workgroup's; -1: a higher channel, -2: a lower one, -3: none
-  auto key_of = [&](float type, float x) -> int {
+  // key of an atom among this workgroup's; -1: a higher channel, -2: a lower one, -3: none.
+  // An atom whose radius is not positive (or not a number) reaches no voxel (its index box,
+  // src/grid_maker.cu:66-79, is empty) and drops out like an atom without a channel.
+  auto key_of = [&](float type, float x, float ar) -> int {
     const float tf = floorf(type);
-    if (!(tf >= 0.f && tf < (float)ntypes)) return -3;
+    if (!(tf >= 0.f && tf < (float)ntypes) || !(ar > 0.f)) return -3;
     const int c = (int)tf;
     if (c < c0) return -2;
     if (c >= c1) return -1;
     return (c - c0) * nxs + (int)slab_of(x, ox, inv_slab, nxs);
   };
 
+  auto scaled = [&](float radius) -> float {
+#pragma clang fp contract(off)
+    return radius * radius_scale;
+  };
   // the atoms of this thread, read once when they fit its registers
   int c_key[kCached];
   float c_x[kCached], c_y[kCached], c_z[kCached], c_r[kCached];
@@ -181,14 +187,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
 #pragma clang fp contract(off)
         c_r[k] = c_r[k] * radius_scale;
       }
-      c_key[k] = have ? key_of(c_t[k], c_x[k]) : -3;
+      c_key[k] = have ? key_of(c_t[k], c_x[k], c_r[k]) : -3;
       if (c_key[k] != -3) my_rmax = fmaxf(my_rmax, c_r[k]);
       my_below += c_key[k] == -2 ? 1 : 0;
     }
   } else {
     for (int a = wb + lane; a < we; a += kWave) {
-      const int key = key_of(types[a], coords[3 * a]);
-      if (key != -3) my_rmax = fmaxf(my_rmax, radii[a] * radius_scale);
+      const float ar = scaled(radii[a]);
+      const int key = key_of(types[a], coords[3 * a], ar);
+      if (key != -3) my_rmax = fmaxf(my_rmax, ar);
       my_below += key == -2 ? 1 : 0;
     }
   }
@@ -227,7 +234,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
 #pragma unroll
     for (int k = 0; k < kCached; ++k) count(c_key[k]);
   } else {
-    for (int a = wb + lane; a < we; a += kWave) count(key_of(types[a], coords[3 * a]));
+    for (int a = wb + lane; a < we; a += kWave)
+      count(key_of(types[a], coords[3 * a], scaled(radii[a])));
   }
   __syncthreads();
   const int slot = off != nullptr ? s_rank : e;
@@ -316,12 +324,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
       const int a = a0 + lane;
       const int ac = a < we ? a : we - 1;
       const float x = coords[3 * ac];
-      float ar;
-      {
-#pragma clang fp contract(off)
-        ar = radii[ac] * radius_scale;
-      }
-      scatter(a < we ? key_of(types[ac], x) : -3, x, coords[3 * ac + 1], coords[3 * ac + 2], ar);
+      const float ar = scaled(radii[ac]);
+      scatter(a < we ? key_of(types[ac], x, ar) : -3, x, coords[3 * ac + 1], coords[3 * ac + 2], ar);
     }
   }
 }
@@ -364,7 +368,7 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
   const float inv_block = 0.25f / g.resolution;             // blocks per unit length along z
   const __amdgpu_buffer_rsrc_t rec_buf = buffer_of(records, (size_t)capacity * 16);
   auto load_round = [&](int first) -> v4u {
-    return __builtin_amdgcn_raw_buffer_load_b128(rec_buf, (first + lane) * 16, 0, 0);
+    return __builtin_amdgcn_raw_buffer_load_b128(rec_buf, (int)((unsigned)(first + lane) * 16u), 0, 0);
   };
 
   // which item: channel range fastest, then the territory, then the example's slot

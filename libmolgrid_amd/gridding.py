@@ -344,6 +344,77 @@ def _ptr(t):
 # --------------------------------------------------------------------------- #
 # Transform
 # --------------------------------------------------------------------------- #
+def _qmul(p, q):
+    """Hamilton product of (arrays of) float32 quaternion components, every product and sum
+    rounded to float32 in the order of include/libmolgrid/quaternion.h:82-91."""
+    a, b, c, d = p
+    ar, br, cr, dr = q
+    return (+a * ar - b * br - c * cr - d * dr,
+            +a * br + b * ar + c * dr - d * cr,
+            +a * cr - b * dr + c * ar + d * br,
+            +a * dr + b * cr - c * br + d * ar)
+
+
+def _qrotate(q, x, y, z):
+    """q * (0, x, y, z) * (conj(q) / norm(q)) on float32 arrays (quaternion.h:145-149)."""
+    a, b, c, d = q
+    n = a * a + b * b + c * c + d * d
+    cj = (a / n, -b / n, -c / n, -d / n)
+    r = _qmul(_qmul(q, (np.zeros_like(x), x, y, z)), cj)
+    return r[1], r[2], r[3]
+
+
+def _host_transform(tr, inverse, src, dst, dotranslate):
+    """Transform.forward / backward for host arrays, on the host (src/transform.cpp:57-108):
+    numpy float32 arithmetic, one rounding per operation, in the reference's order -- the same
+    floats the device kernel stores.  float64 arrays are narrowed where the reference narrows
+    them (at the call of Quaternion::transform / rotate, which take floats)."""
+    def view(x, out):
+        x = _unwrap(x)
+        if isinstance(x, torch.Tensor):
+            if x.dtype not in (torch.float32, torch.float64):
+                raise ValueError("only float32 and float64 tensors are supported")
+            if not x.is_contiguous():
+                raise ValueError("tensor is not contiguous")
+            return x.detach().numpy()
+        if out:
+            if not (isinstance(x, np.ndarray) and x.dtype in (np.float32, np.float64)
+                    and x.flags.c_contiguous and x.flags.writeable):
+                raise ValueError("out: output must be a writable C-contiguous float32 array")
+            return x
+        x = np.asarray(x)
+        return x if x.dtype == np.float64 else np.ascontiguousarray(x, dtype=np.float32)
+
+    a_in, a_out = view(src, False), view(dst, True)
+    if a_in.ndim != 2 or a_out.ndim != 2:
+        raise ValueError("expected 2 dimensions")
+    # transform.h:131-146 (checkGrids)
+    if a_in.shape[0] != a_out.shape[0]:
+        raise ValueError("Different dimensions and input and output coordinates grids.")
+    if a_in.shape[1] != 3:
+        raise ValueError("Input coordinates wrong dimension.")
+    if a_out.shape[1] != 3:
+        raise ValueError("Output coordinates are wrong dimension.")
+    q = tuple(_f32(v) for v in tr.Q.as_tuple())
+    c = [_f32(v) for v in tr.center]
+    t = [_f32(v) if dotranslate else _f32(0.0) for v in tr.translate]
+    with np.errstate(all="ignore"):
+        if not inverse:
+            x, y, z = (a_in[:, k].astype(np.float32) - c[k] for k in range(3))
+            r = _qrotate(q, x, y, z)
+            res = [r[k] + c[k] + t[k] for k in range(3)]
+        else:
+            n = q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3]
+            qinv = (q[0] / n, -q[1] / n, -q[2] / n, -q[3] / n)
+            un = [-t[k] - c[k] for k in range(3)]
+            # the sum is formed in the array's own type, then narrowed (transform.cpp:97-99)
+            x, y, z = ((a_in[:, k] + un[k]).astype(np.float32) for k in range(3))
+            r = _qrotate(qinv, x, y, z)
+            res = [r[k] + c[k] for k in range(3)]
+    for k in range(3):
+        a_out[:, k] = res[k]
+
+
 class Transform(object):
     """Rigid transform: rotate about ``center`` by ``Q``, then translate.
 
@@ -414,6 +485,11 @@ class Transform(object):
             if src.coords.shape[0] != dst.coords.shape[0]:
                 raise ValueError("Incompatible coordinateset sizes")
             src, dst = src.coords, dst.coords
+        if _is_host(src) and _is_host(dst):
+            # the reference's Grid<Dtype, 2, false> overloads (src/transform.cpp:57-108) run on
+            # the host; so do these, with the same float arithmetic as the kernel
+            _host_transform(self, fn is _lib.mg_transform_backward, src, dst, dotranslate)
+            return
         same = dst is src
         a_in = _Arg(src, "in", 2, wide=True)
         a_out = a_in if same and a_in.t is not None else _Arg(dst, "out", 2, out=True, wide=True)
@@ -1056,7 +1132,8 @@ class GridMaker(object):
             need = int(_lib.mg_forward_index_workspace_size(p, B, n, T))
             ws = None
             if need:
-                key = ("forward_index_ws", torch.cuda.current_device())
+                # one workspace per device AND stream: calls on two streams may overlap
+                key = ("forward_index_ws", torch.cuda.current_device(), stream)
                 ws = batch.scratch.get(key) if batch is not None else None
                 if ws is None or ws.numel() < need:
                     ws = torch.empty(need, dtype=torch.uint8, device=_device())

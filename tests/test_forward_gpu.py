@@ -90,6 +90,28 @@ def test_unusual_radius_multiples(mg, gm_args):
         assert_close(got, ref, what="forward")
 
 
+@pytest.mark.parametrize("binary", [False, True])
+def test_zero_and_negative_radii_add_nothing(mg, binary):
+    """An atom whose radius is zero or negative has an empty index box in the reference
+    (src/grid_maker.cu:66-79): it adds nothing, whatever its neighbours are."""
+    rng = np.random.default_rng(21)
+    coords, types, radii = synth.small_index_case(rng, 120, 3, 6.0)
+    radii[::3] = 0.0
+    radii[1::3] = -radii[1::3]
+    keep = radii > 0
+    gm_args = (0.5, 11.5, binary)
+    ref = oracle.GridMaker(*gm_args).forward((0, 0, 0), coords, types, radii, 3)
+    only = oracle.GridMaker(*gm_args).forward((0, 0, 0), coords[keep], types[keep], radii[keep], 3)
+    assert np.array_equal(ref, only)                       # the oracle itself: nothing added
+    got = gpu_forward(mg, gm_args, (0, 0, 0), coords, types, radii, 3)
+    got_only = gpu_forward(mg, gm_args, (0, 0, 0), coords[keep], types[keep], radii[keep], 3)
+    assert np.array_equal(got, got_only)
+    if binary:
+        assert np.array_equal(got, ref)
+    else:
+        assert_close(got, ref, what="forward")
+
+
 def test_many_atoms_on_one_spot(mg):
     """More candidates than one LDS list holds: 3000 atoms inside one tile."""
     rng = np.random.default_rng(3)
@@ -99,7 +121,8 @@ def test_many_atoms_on_one_spot(mg):
     radii = rng.uniform(1.0, 1.5, n).astype(np.float32)
     ref = oracle.GridMaker(0.5, 7.5).forward((0, 0, 0), coords, types, radii, 2)
     got = gpu_forward(mg, (0.5, 7.5), (0, 0, 0), coords, types, radii, 2)
-    # thousands of terms per voxel: same summation order, so still tight
+    # thousands of terms per voxel, summed by the kernel in record order (x slab of the atom's
+    # centre, then atom number) and by the oracle in atom order: equal to rounding
     assert_close(got, ref, what="dense forward")
 
 

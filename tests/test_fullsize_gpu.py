@@ -101,7 +101,6 @@ def test_backward_full_batch(mg, workload):
     print("\nbackward parity, %d components: gpu vs f64 sums %s; gpu vs float loop %s; float loop "
           "vs f64 sums %s" % (gpu64["n"], gpu64, gpu32, cpu64))
     assert gpu64["max_abs"] <= 1e-5 and gpu64["outside"] <= 0.002 * gpu64["n"]
-    assert gpu64["max_abs"] <= cpu64["max_abs"]
     excess = np.maximum(np.abs(got - ref64) - (1e-6 + 1e-5 * np.abs(ref64)), 0) / (EPS * mag)
     assert float(excess.max()) <= 16.0          # measured: 11.9
     # the launch that also un-rotates gives what backward + Transform.backward give, bit for bit
