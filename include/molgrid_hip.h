@@ -104,8 +104,14 @@ int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per
  * `out` is overwritten completely (no memset needed before the call).  Two
  * launches: the atoms are sorted by channel into `workspace` (device memory,
  * at least mg_forward_index_workspace_size() bytes, 256-byte aligned, contents
- * undefined before and after), then splatted.  Calls that run concurrently need
- * a workspace each.  MG_ERR_UNSUPPORTED: a channel of 4 GB or more, or
+ * undefined before and after; a pointer that is not 256-byte aligned is
+ * MG_ERR_INVALID_ARGUMENT), then splatted.  Calls that run concurrently need a
+ * workspace each.  `atoms_per_example` sizes the workspace and must be at least
+ * the largest example's atom count, also with `atom_offsets`: atoms of an
+ * example beyond it are left out of the grid without an error, and 0 means "no
+ * atoms at all" (the offsets and arrays are then not looked at).  An atom whose
+ * radius * radius_scale is not positive adds nothing, like an atom with a negative
+ * type.  MG_ERR_UNSUPPORTED: a channel of 4 GB or more, or
  * nbatch * atoms_per_example >= 2^28. */
 int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                         int atoms_per_example, const float* grid_centers,
@@ -118,12 +124,16 @@ int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
 size_t mg_forward_index_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
                                        int ntypes);
 
-/* The same with a workspace that the library keeps per device: it is allocated
- * (hipMalloc) by the first call on a device and replaced (hipFree + hipMalloc,
- * which wait for the device) when a call needs a larger one; it is never
- * released.  All calls on one device share it, so calls on different streams of
- * one device must not overlap.  Callers that must not allocate, or that use
- * several streams, take mg_forward_index_ws. */
+/* The same with a workspace that the library keeps per device and stream: it is
+ * allocated (hipMalloc) by the first call on a stream, and a call that needs
+ * more gets a new, larger block while the old one stays allocated (launches
+ * already enqueued may still use it); nothing is released before the process
+ * ends.  Safe for several host threads and several streams: a lock is held
+ * until both launches are enqueued, calls on one stream follow each other in
+ * that stream, calls on different streams use different blocks (up to 256
+ * device/stream pairs, then MG_ERR_UNSUPPORTED).  Callers that must not
+ * allocate (HIP graph capture) take mg_forward_index_ws or
+ * mg_forward_index_static. */
 int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                      int atoms_per_example, const float* grid_centers,
                      const float grid_center_host[3], const float* coords,

@@ -56,7 +56,11 @@ def _load():
         raise ImportError(
             "%s is missing: build it with `python libmolgrid_amd/build.py` "
             "(the gridding kernels have no CPU fallback)" % LIB_PATH)
-    lib = ctypes.CDLL(LIB_PATH)
+    return declare(ctypes.CDLL(LIB_PATH))
+
+
+def declare(lib):
+    """Argument and result types of every entry point of include/molgrid_hip.h on a loaded library."""
     gm = ctypes.POINTER(mg_gridmaker)
     lib.mg_version.restype = _i
     lib.mg_error_string.restype = ctypes.c_char_p

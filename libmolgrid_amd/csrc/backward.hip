@@ -65,11 +65,7 @@ __device__ __forceinline__ float point_density(const GridArg& g, float dx, float
 constexpr int kRawBufferFlags = 0x00020000;   // untyped 32-bit elements, no swizzle (gfx9 family)
 
 // a * b with 0 * anything = 0 (also infinities and NaNs)
-__device__ __forceinline__ float mul_zero_wins(float a, float b) {
-  float r;
-  asm("v_mul_legacy_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
+__device__ __forceinline__ float mul_zero_wins(float a, float b) { return mul_legacy(a, b); }
 
 // Voxel range [lo, lo + n) along one axis whose centres lie within `reach` of `coord` (n <= 0:
 // none).  Tighter than the reference's index box (src/grid_maker.cu:66-79), which adds a voxel

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "gfx950_asm.h"
 #include "molgrid_hip.h"
 
 namespace mg {

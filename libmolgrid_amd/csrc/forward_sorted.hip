@@ -362,7 +362,7 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
     st_rel[k] = (unsigned)((st_rx[k] * dim + st_ry[k]) * dim + st_z[k]) * 4u;
   }
   float quad_c = g.C;
-  asm volatile("" : "+v"(quad_c));          // vector register (an fma takes one scalar operand)
+  keep_in_vgpr(quad_c);
   const float frm2 = uniform(g.frm * g.frm);
   const float grm2 = uniform(g.grm * g.grm);
   const float inv_block = 0.25f / g.resolution;             // blocks per unit length along z
@@ -613,8 +613,10 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
       if (y0 + col * kColXY >= dim) break;
       const bool from_stage = (touched >> col) & 1u;
       if (from_stage) {
+        wave_lds_fence();                      // the previous column has been read
 #pragma unroll
         for (int q = 0; q < kBlocks; ++q) stage[stage_lane + q * 4] = acc[col][q];
+        wave_lds_fence();
       }
       store_column(c, col, from_stage);
     }

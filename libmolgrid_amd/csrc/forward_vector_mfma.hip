@@ -64,9 +64,6 @@ constexpr int kRowsBytes = (kRecChunk + 1) * kRowBytes;   // the last row belong
 __device__ __forceinline__ float uniform(float v) {
   return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
 }
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
 
 template <bool BINARY>
 __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void
