@@ -155,6 +155,15 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
                             const float* type_index, const float* radii, int ntypes, float* out,
                             void* stream);
 
+/* No counterpart in the reference.  Selects the write-out of the splat launch of
+ * mg_forward_index* for grids of at most 48 voxels a side whose rows are whole
+ * 16-byte pieces (dim % 4 == 0, `out` 16-byte aligned): 1 = one workgroup per
+ * (example, channel, slab of four x planes) that gathers the sums of its waves
+ * in LDS and writes the slab as whole 4 KB pages, 0 = one wave per territory
+ * writing its own rows.  The grids are the same bit for bit.  Process-wide;
+ * returns the previous setting. */
+int mg_forward_index_paged(int on);
+
 /* GridMaker::forward, vector types; replaces forward_gpu_vec and its launcher
  * (src/grid_maker.cu:348-441), values of src/grid_maker.cpp:214-271.
  *   type_vector [n, ntypes]; radii [n], or [nbatch, ntypes] when

@@ -19,7 +19,7 @@ MG_STATIC_SCRATCH_BYTES = 16 << 20
 EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
-    "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_vector", "mg_backward_index",
+    "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_index_paged", "mg_forward_vector", "mg_backward_index",
     "mg_backward_index_unrotated",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate", "mg_interpolate_force_gather",
     "mg_narrow", "mg_widen",
@@ -90,6 +90,7 @@ def declare(lib):
     lib.mg_narrow.argtypes = [_vp, _vp, ctypes.c_size_t, _vp]
     lib.mg_widen.argtypes = [_vp, _vp, ctypes.c_size_t, _vp]
     lib.mg_interpolate_force_gather.argtypes = [_i]
+    lib.mg_forward_index_paged.argtypes = [_i]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)
         if name not in ("mg_error_string", "mg_forward_index_workspace_size"):

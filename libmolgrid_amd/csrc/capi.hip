@@ -324,6 +324,8 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
                             MG_STATIC_SCRATCH_BYTES, stream);
 }
 
+int mg_forward_index_paged(int on) { return set_forward_paged(on); }
+
 int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                       int atoms_per_example, const float* grid_centers,
                       const float grid_center_host[3], const float* coords,

@@ -28,6 +28,7 @@
 // Every global access of the splat kernel goes through buffer instructions that carry the
 // extent of the array they address: an index outside it reads zero or is dropped.
 #include <algorithm>
+#include <atomic>
 
 #include "kernels.h"
 #include "splat_common.h"
@@ -44,6 +45,22 @@ constexpr int kPieces = 16 * (kSlabZ / 4) / kWave;   // float4 pieces of a colum
 constexpr int kBufferFlags = 0x00020000;         // untyped 32-bit elements, no swizzle
 constexpr int kItemChannels = 4;                 // channels an item takes, about
 constexpr int kItemChannelsMax = 64;             // ... and at most (one per lane)
+constexpr int kSortChannels = 4;                 // channels a workgroup of the sort takes, about
+
+// Paged write-out: a workgroup of one wave per pair of columns owns a whole slab of four x planes
+// of ONE channel -- a contiguous run of the output -- collects the sums of its waves in LDS and
+// writes the run as bursts of whole 4 KB pages, each page by one wave in four back-to-back
+// stores.  For grids of up to kPagedDim voxels a side, whose slab fits the LDS.
+constexpr int kPagedDim = 48;
+constexpr int kPagedWaves = (kPagedDim + 2 * kColXY - 1) / (2 * kColXY);   // 6
+constexpr int kPageBytes = 4096;
+// LDS slab [4 planes][dim rows][dim + 4]: rows padded by four floats and planes spaced 16 banks
+// (mod 32) apart, so that the 32 lanes of a half wave (2 planes x 4 rows x 4 voxels) hit 32 banks
+__host__ __device__ constexpr int paged_row(int dim) { return dim + 4; }
+__host__ __device__ constexpr int paged_plane(int dim) {
+  return dim * paged_row(dim) + ((16 - dim * paged_row(dim)) % 32 + 32) % 32;
+}
+constexpr int kSlabFloats = kColXY * paged_plane(kPagedDim);               // 10,048 floats
 
 constexpr int kSortWaves = 16;
 constexpr int kSortThreads = kSortWaves * kWave;
@@ -333,14 +350,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
 // ------------------------------------------------------------------------------------------
 // Launch 2
 // ------------------------------------------------------------------------------------------
-template <bool BINARY, bool EXACT, int COLS>
-__global__ __launch_bounds__(kWave) void splat_sorted_kernel(
+template <bool BINARY, bool EXACT, int COLS, bool PAGED>
+__global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sorted_kernel(
     GridArg g, const float4* __restrict__ slot_info, const int* __restrict__ cand,
     const float4* __restrict__ records, int capacity, float* __restrict__ out,
     int nxs, int nyp, int nzs, int nranges, int aligned_rows, int slab_z) {
-  __shared__ __align__(16) float stage[kPlane];
+  // one column of one wave (rows padded), or the workgroup's slab of four x planes
+  __shared__ __align__(16) float stage[PAGED ? kSlabFloats : kPlane];
 
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
   const int dim = g.dim;
   const int ntypes = g.ntypes;
   const size_t chan_stride = (size_t)dim * dim * dim;   // the host has checked: < 2^30 floats
@@ -371,16 +389,28 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
     return __builtin_amdgcn_raw_buffer_load_b128(rec_buf, (int)((unsigned)(first + lane) * 16u), 0, 0);
   };
 
-  // which item: channel range fastest, then the territory, then the example's slot
+  // which item: channel range fastest, then the territory, then the example's slot; paged:
+  // the x slab fastest, then the channel (consecutive workgroups write consecutive runs of the
+  // output), the wave of the workgroup is the pair of columns
   int t = blockIdx.x;
-  const int range = t % nranges;
-  t /= nranges;
-  const int yp = t % nyp;
-  t /= nyp;
-  const int zs = t % nzs;
-  t /= nzs;
-  const int xs = t % nxs;
-  const int slot = t / nxs;
+  int range, yp, zs, xs, slot;
+  if (PAGED) {
+    xs = t % nxs;
+    t /= nxs;
+    range = t % nranges;
+    slot = t / nranges;
+    yp = threadIdx.x >> 6;
+    zs = 0;
+  } else {
+    range = t % nranges;
+    t /= nranges;
+    yp = t % nyp;
+    t /= nyp;
+    zs = t % nzs;
+    t /= nzs;
+    xs = t % nxs;
+    slot = t / nxs;
+  }
   const int nmine = (ntypes - range + nranges - 1) / nranges;   // channels range, range + R, ...
   if (nmine <= 0) return;
 
@@ -431,6 +461,40 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
     }
   };
 
+  // Paged: the slab of channel c -> global memory, whole 4 KB pages (by their address), a page
+  // per wave in four back-to-back stores; from the LDS slab or as zeros.
+  auto store_pages = [&](int c, bool from_slab) {
+    float* const chan = out_e + (size_t)c * chan_stride;
+    const __amdgpu_buffer_rsrc_t out_buf = buffer_of(chan, chan_stride * 4);
+    const unsigned plane_bytes = (unsigned)(dim * dim) * 4u;
+    const unsigned first = (unsigned)x0 * plane_bytes;                  // of the slab, in the channel
+    const unsigned bytes = (unsigned)(min(x0 + kColXY, dim) - x0) * plane_bytes;
+    // bytes from the slab's start back to the page boundary at or before it
+    const unsigned lead = (unsigned)((reinterpret_cast<uintptr_t>(chan) + first) & (kPageBytes - 1));
+    const int npages = (int)((lead + bytes + kPageBytes - 1) / kPageBytes);
+    const float inv_pieces = 4.0f / (float)dim, inv_dim = 1.0f / (float)dim;
+    const int prow = paged_row(dim), pplane = paged_plane(dim);
+    for (int page = (int)(threadIdx.x >> 6); page < npages; page += (int)(blockDim.x >> 6)) {
+#pragma unroll
+      for (int k = 0; k < kPageBytes / (kWave * 16); ++k) {
+        // byte of this lane's piece relative to the slab's start
+        const int rel = page * kPageBytes + (k * kWave + lane) * 16 - (int)lead;
+        if (rel >= 0 && rel < (int)bytes) {
+          v4f v = {0.f, 0.f, 0.f, 0.f};
+          if (from_slab) {
+            const int piece = rel >> 4;
+            const int row = (int)(((float)piece + 0.5f) * inv_pieces);   // piece / (dim / 4)
+            const int px = (int)(((float)row + 0.5f) * inv_dim);         // row / dim
+            v = *reinterpret_cast<const v4f*>(stage + px * pplane + (row - px * dim) * prow +
+                                              (piece * 4 - row * dim));
+          }
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf,
+                                                 (int)(first + (unsigned)rel), 0, 2);
+        }
+      }
+    }
+  };
+
   unsigned long long full = __ballot(lane < nmine && se.y > se.x);    // my channels with atoms
   unsigned long long empty = __ballot(lane < nmine && se.y <= se.x);  // and without
   v4u pre = {0u, 0u, 0u, 0u};
@@ -440,8 +504,12 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
   while (empty != 0) {
     const int j = __builtin_ctzll(empty);
     empty &= empty - 1ull;
+    if (PAGED) {
+      store_pages(range + j * nranges, false);
+    } else {
 #pragma unroll
-    for (int col = 0; col < COLS; ++col) store_column(range + j * nranges, col, false);
+      for (int col = 0; col < COLS; ++col) store_column(range + j * nranges, col, false);
+    }
   }
   if (full == 0) return;
 
@@ -606,6 +674,26 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
       }
     }
 
+    if (PAGED) {
+      // sums -> the workgroup's slab (every wave its own rows; voxels outside the grid have no
+      // place in it), then the slab -> pages.  All waves of the workgroup have the same channels
+      // with atoms (one table entry serves them all), so they meet at the barriers.
+      const int prow = paged_row(dim), pplane = paged_plane(dim);
+#pragma unroll
+      for (int col = 0; col < COLS; ++col) {
+        const int y = y0 + col * kColXY + ly;
+        if (vxi < dim && y < dim) {
+          float* const dst = stage + lx * pplane + y * prow + lz;
+#pragma unroll
+          for (int q = 0; q < kBlocks; ++q)
+            if (q * 4 + lz < dim) dst[q * 4] = acc[col][q];
+        }
+      }
+      lds_barrier();
+      store_pages(c, true);
+      if (full != 0) lds_barrier();            // the slab is written again for the next channel
+      continue;
+    }
     // write-out, column by column: sums -> the stage -> z rows (or zeros straight away); LDS
     // keeps the order of one wave's accesses, so no barrier is involved
 #pragma unroll
@@ -621,6 +709,26 @@ __global__ __launch_bounds__(kWave) void splat_sorted_kernel(
       store_column(c, col, from_stage);
     }
   }
+}
+
+// Whether the paged write-out serves this grid: whole float4 pieces in a row, one z slab, a slab of
+// four x planes that fits the LDS.
+bool paged_serves(const GridArg& g, const float* out) {
+  return g.dim % 4 == 0 && g.dim <= kPagedDim && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+}
+
+template <bool BINARY>
+hipError_t launch_splat_paged(const GridArg& g, const SortedAtoms& s, int nbatch, float* out,
+                              hipStream_t stream) {
+  const int dim = g.dim;
+  const int nxs = (dim + kColXY - 1) / kColXY;
+  const int nyp = (dim + 2 * kColXY - 1) / (2 * kColXY);      // waves of a workgroup, <= kPagedWaves
+  const long long nitems = (long long)nbatch * nxs * g.ntypes;
+  if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, false, 2, true>), dim3((unsigned)nitems),
+                     dim3(nyp * kWave), 0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out,
+                     nxs, nyp, 1, g.ntypes, 1, kSlabZ);
+  return hipGetLastError();
 }
 
 template <bool BINARY, bool EXACT, int COLS>
@@ -640,11 +748,14 @@ hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, floa
   const long long nitems = (long long)nbatch * nxs * nzs * nyp * nranges;
   if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
   const int aligned = ((dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
-  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS>), dim3((unsigned)nitems), dim3(kWave),
+  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS, false>), dim3((unsigned)nitems), dim3(kWave),
                      0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out, nxs, nyp, nzs,
                      nranges, aligned, slab_z);
   return hipGetLastError();
 }
+
+// 1: grids that the paged write-out serves take it
+std::atomic<int> g_paged{0};
 
 }  // namespace
 
@@ -673,7 +784,7 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
   if ((long long)g.ntypes * nxs >= (1 << 26)) return hipErrorInvalidValue;
   const SortedAtoms s = carve(workspace, nbatch, g.ntypes * nxs, capacity);
   // channels per workgroup of the sort: a few, and no more keys than it handles
-  const int per_part = std::max(1, std::min(kItemChannels, kKeyGroup / nxs));
+  const int per_part = std::max(1, std::min(kSortChannels, kKeyGroup / nxs));
   const int parts = (g.ntypes + per_part - 1) / per_part;
   hipLaunchKernelGGL(sort_atoms_kernel, dim3((unsigned)(parts * nbatch)), dim3(kSortThreads), 0, stream, g,
                      batch, nbatch, nxs, parts, per_part, binary ? 1.0f : g.frm, centers, coords,
@@ -685,8 +796,14 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
     if (binary) return launch_splat<true, true, 1>(g, s, nbatch, out, stream);
     return launch_splat<false, true, 1>(g, s, nbatch, out, stream);
   }
+  if (g_paged.load(std::memory_order_relaxed) != 0 && paged_serves(g, out)) {
+    if (binary) return launch_splat_paged<true>(g, s, nbatch, out, stream);
+    return launch_splat_paged<false>(g, s, nbatch, out, stream);
+  }
   if (binary) return launch_splat<true, false, 2>(g, s, nbatch, out, stream);
   return launch_splat<false, false, 2>(g, s, nbatch, out, stream);
 }
+
+int set_forward_paged(int on) { return g_paged.exchange(on ? 1 : 0); }
 
 }  // namespace mg

@@ -37,6 +37,12 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
                                  bool binary, bool exact, void* workspace, size_t workspace_bytes,
                                  hipStream_t stream);
 
+// Which write-out the splat launch uses for grids of up to 48 voxels a side with rows of whole
+// float4 pieces: 1 = workgroups that own a slab of four x planes of one channel and write it as
+// whole 4 KB pages, 0 = one wave per territory writing its own rows.  Same grids bit for bit.
+// Returns the previous setting.
+int set_forward_paged(int on);
+
 // vector types with per-atom radii, density mode, on the matrix cores (forward_vector_mfma.hip)
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
                                       const Vec3Arg& centers, const float* coords,

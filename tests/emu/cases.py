@@ -172,6 +172,52 @@ def group_forward_batch():
     _checked[0] += 1
 
 
+def group_forward_paged():
+    """The paged write-out (workgroups that own a slab and write whole 4 KB pages) gives the grids
+    of the per-wave write-out bit for bit: dims 16, 24, 48 and smaller, binary and Gaussian, batches
+    with empty examples, output arrays at several alignments inside a 4 KB page."""
+    lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    shapes = [(1.0, 15.0, 40, 200), (0.25, 5.75, 2, 15), (0.5, 23.5, 28, 300), (0.5, 3.5, 3, 12),
+              (0.5, 1.5, 2, 5), (0.5, 21.5, 5, 150)]
+    for res, dimension, ntypes, natoms in shapes:
+        for binary in (False, True):
+            rng = np.random.default_rng(31 + natoms)
+            coords, types, radii = synth.small_index_case(rng, natoms, ntypes, dimension / 2 + 2.0)
+            center = rng.uniform(-1, 1, 3).astype(np.float32)
+            ref = oracle.GridMaker(res, dimension, binary).forward(center, coords, types, radii, ntypes)
+            assert lib.mg_forward_index_paged(0) in (0, 1)
+            plain = forward_index((res, dimension, binary), center, coords, types, radii, ntypes).copy()
+            lib.mg_forward_index_paged(1)
+            paged = forward_index((res, dimension, binary), center, coords, types, radii, ntypes)
+            lib.mg_forward_index_paged(0)
+            what = "paged %s binary=%s" % ((res, dimension, ntypes, natoms), binary)
+            close(paged, plain, what + " vs per-wave write-out", exact=True)
+            close(paged, ref, what + " vs oracle", exact=binary)
+    # a ragged batch with an empty example; the output at offsets of 16, 1040 and 4080 bytes from
+    # a page boundary (pages are taken by address)
+    cfg = synth.index_batch(2, 4, (30, 120), (3, 9), ntypes=6)
+    off = np.array([0, 40, 40, 130, 200], np.int64)
+    gm = oracle.GridMaker(0.5, 11.5)
+    ref = gm.forward_batch(off, cfg["centers"], cfg["coords"][:200], cfg["types"][:200],
+                           cfg["radii"][:200], 6)
+    g = E.gridmaker(0.5, 11.5)
+    dim = int(g.dim)
+    nfl = 4 * 6 * dim ** 3
+    need = lib.mg_forward_index_workspace_size(ctypes.byref(g), 4, 90, 6)
+    ws = E.array(need, np.uint8, tight=False)
+    args = [E.ptr(E.put(off, np.int32)), 90, E.ptr(E.put(cfg["centers"])), E.f3((0, 0, 0)),
+            E.ptr(E.put(cfg["coords"][:200])), E.ptr(E.put(cfg["types"][:200])),
+            E.ptr(E.put(cfg["radii"][:200])), 6]
+    lib.mg_forward_index_paged(1)
+    for shift in (4, 260, 1020):
+        big = E.array(nfl + shift, fill=7.0)
+        out = big[shift:]
+        assert lib.mg_forward_index_ws(ctypes.byref(g), 4, *args, out.ctypes.data, E.ptr(ws), need, None) == 0
+        close(out.reshape(ref.shape), ref, "paged, output %d bytes into its page" % (4 * shift))
+        assert np.all(big[:shift] == 7.0)
+    lib.mg_forward_index_paged(0)
+
+
 GROUPS = {k[len("group_"):]: v for k, v in list(globals().items()) if k.startswith("group_")}
 
 if __name__ == "__main__":

@@ -24,7 +24,7 @@ def emulated_library():
     return build_emu.build()
 
 
-@pytest.mark.parametrize("group", ["transform", "forward_index", "forward_batch"])
+@pytest.mark.parametrize("group", ["transform", "forward_index", "forward_batch", "forward_paged"])
 def test_group(emulated_library, group):
     p = subprocess.run([sys.executable, RUNNER, group], stdout=subprocess.PIPE,
                        stderr=subprocess.STDOUT, text=True, timeout=1200)
