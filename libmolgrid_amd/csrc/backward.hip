@@ -173,6 +173,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
 
           // one pass: lanes below `count` take the columns cols[0 .. count)
           auto march = [&](int count) {
+            wave_lds_fence();                    // the list is complete
             const bool live = lane < count;
             const int packed = cols[live ? lane : 0];
             const int j = packed >> 16, k = packed & 0xffff;
@@ -222,6 +223,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
 
           int pending = 0;
           for (int c0 = 0; c0 < ncols; c0 += kWave) {
+            wave_lds_fence();                    // the entries moved to the front have been read
             const int cand = c0 + lane;
             const int j = (int)(((float)cand + 0.5f) * inv_nk), k = cand - j * nk;
             const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;

@@ -299,6 +299,7 @@ splat_vector_mfma_kernel(
           for (int blk = 0; blk < kBlocksPerWave; ++blk)
             if (lane < 24) s_mini[wave][blk][nlist[blk] + lane] = (unsigned short)(kRecChunk * kRowBytes);
 
+          wave_lds_fence();                    // the wave's lists are complete
           __builtin_amdgcn_s_setprio(0);
 #pragma unroll
           for (int blk = 0; blk < kBlocksPerWave; ++blk) {

@@ -126,7 +126,9 @@ __global__ __launch_bounds__(kTileThreads) void interpolate_tiled_kernel(
 
   // ---- window of the tile: bounding box of the images of its eight corners -----------------
   for (int r = tid; r < kRowsPad; r += kTileThreads) s_rowmask[r] = 0u;
-  if (tid < 8) {
+  {
+    // (every group of eight lanes does this, so that the shuffles are not inside a branch;
+    // thread 0 publishes the result)
     const int ci = min(tx * kTileX + ((tid >> 2) & 1) * (kTileX - 1), od - 1);
     const int cj = min(ty * kTileY + ((tid >> 1) & 1) * (kTileY - 1), od - 1);
     const int ck = min(tz * kTileZ + (tid & 1) * (kTileZ - 1), od - 1);

@@ -218,6 +218,204 @@ def group_forward_paged():
     lib.mg_forward_index_paged(0)
 
 
+EPS = float(np.finfo(np.float32).eps)
+
+
+def check_grads(got, ref32, ref64, mag, what):
+    """The bounds of tests/test_backward_gpu.py."""
+    _checked[0] += 1
+    got = np.asarray(got, np.float64)
+    bound64 = ATOL + RTOL * np.abs(ref64) + 16 * EPS * mag
+    err64 = np.abs(got - ref64)
+    assert (err64 <= bound64).all(), "%s vs f64 oracle: worst excess %g" % (what, float((err64 - bound64).max()))
+    bound32 = ATOL + RTOL * np.abs(ref32) + 64 * EPS * mag
+    err32 = np.abs(got - ref32.astype(np.float64))
+    assert (err32 <= bound32).all(), "%s vs f32 oracle: worst excess %g" % (what, float((err32 - bound32).max()))
+
+
+def group_backward_index():
+    for res, dimension, ntypes, natoms in [(0.5, 6.0, 3, 20), (0.5, 12.0, 5, 60), (0.25, 5.75, 2, 15),
+                                           (0.5, 23.5, 28, 200)]:
+        rng = np.random.default_rng(21 + natoms)
+        coords, types, radii = synth.small_index_case(rng, natoms, ntypes, dimension / 2 + 2.0)
+        types = types + rng.uniform(-0.4, 0.4, natoms).astype(np.float32) * (types >= 0)
+        radii[0] = 0.0                                   # an atom without extent: zero gradient
+        center = rng.uniform(-1, 1, 3).astype(np.float32)
+        og = oracle.GridMaker(res, dimension)
+        diff = rng.standard_normal(og.grid_shape(ntypes)).astype(np.float32)
+        ref32 = og.backward(center, coords, types, radii, diff)
+        ref64 = og.backward(center, coords, types, radii, diff, f64=True)
+        mag = np.abs(og.backward(center, coords, types, radii, np.abs(diff), f64=True)).max(
+            axis=1, keepdims=True) + 1e-30
+        g = E.gridmaker(res, dimension)
+        grads = E.array((natoms, 3), fill=9.0)
+        c, t, r, d = E.put(coords), E.put(types), E.put(radii), E.put(diff)
+        assert lib.mg_backward_index(ctypes.byref(g), 1, None, natoms, None, E.f3(center), E.ptr(c),
+                                     E.ptr(t), E.ptr(r), ntypes, E.ptr(d), E.ptr(grads), None) == 0
+        check_grads(grads, ref32, ref64, mag, "backward %s" % ((res, dimension, ntypes, natoms),))
+        assert np.all(grads[np.round(types) < 0] == 0) and np.all(grads[0] == 0)
+        # the launch that also un-rotates = backward + Transform.backward(dotranslate=False)
+        q = rng.normal(size=4).astype(np.float32)
+        rc = rng.uniform(-2, 2, 3).astype(np.float32)
+        un = E.array((natoms, 3), fill=9.0)
+        assert lib.mg_backward_index_unrotated(ctypes.byref(g), 1, None, natoms, None, E.f3(center),
+                                               E.ptr(c), E.ptr(t), E.ptr(r), ntypes, E.ptr(d), None,
+                                               E.f4(q), None, E.f3(rc), E.ptr(un), None) == 0
+        close(un, oracle.transform_backward(q, rc, np.zeros(3, np.float32), np.array(grads), False),
+              "fused un-rotation", exact=True)
+    # a ragged batch, 10 % of the upstream gradient non-zero
+    cfg = synth.index_batch(2, 4, (60, 200), (5, 20), ntypes=8)
+    off = cfg["offsets"]
+    rng = np.random.default_rng(8)
+    og = oracle.GridMaker(0.5, 15.5)
+    diff = rng.standard_normal((4,) + og.grid_shape(8)).astype(np.float32)
+    diff *= rng.random(diff.shape) < 0.1
+    ref32 = og.backward_batch(off, cfg["centers"], cfg["coords"], cfg["types"], cfg["radii"], diff)
+    g = E.gridmaker(0.5, 15.5)
+    n = int(off[-1])
+    grads = E.array((n, 3), fill=9.0)
+    assert lib.mg_backward_index(ctypes.byref(g), 4, E.ptr(E.put(off, np.int32)),
+                                 int(np.diff(off).max()), E.ptr(E.put(cfg["centers"])),
+                                 E.f3((0, 0, 0)), E.ptr(E.put(cfg["coords"])), E.ptr(E.put(cfg["types"])),
+                                 E.ptr(E.put(cfg["radii"])), 8, E.ptr(E.put(diff)), E.ptr(grads), None) == 0
+    _checked[0] += 1
+    assert np.allclose(grads, ref32, rtol=1e-4, atol=2e-5), float(np.abs(grads - ref32).max())
+
+
+def vector_case(rng, natoms, ntypes, extent, sparse=0.5):
+    coords = rng.uniform(-extent, extent, (natoms, 3)).astype(np.float32)
+    tv = rng.dirichlet(np.full(ntypes, 0.3), natoms) * rng.uniform(0.5, 1.5, (natoms, 1))
+    tv = (tv * (rng.random((natoms, ntypes)) > sparse)).astype(np.float32)
+    radii = rng.uniform(0.8, 2.0, natoms).astype(np.float32)
+    return coords, tv, radii
+
+
+def forward_vector(gm_args, center, coords, tv, radii):
+    g = E.gridmaker(*gm_args)
+    dim, ntypes = int(g.dim), tv.shape[1]
+    out = E.array((ntypes, dim, dim, dim), fill=3.0)
+    code = lib.mg_forward_vector(ctypes.byref(g), 1, None, len(coords), None, E.f3(center),
+                                 E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), ntypes,
+                                 E.ptr(out), None)
+    assert code == 0, code
+    return out
+
+
+def group_forward_vector():
+    """Matrix-core kernel (per-atom radii) and the tile kernel (exact predicates, radii by type)."""
+    for ntypes in (2, 14, 28, 37):
+        for binary in (False, True):
+            rng = np.random.default_rng(100 + ntypes)
+            coords, tv, radii = vector_case(rng, 60, ntypes, 7.0)
+            ref = oracle.GridMaker(0.5, 11.5, binary).forward((0.2, -0.1, 0), coords, tv, radii)
+            got = forward_vector((0.5, 11.5, binary), (0.2, -0.1, 0), coords, tv, radii)
+            close(got, ref, "vector forward T=%d binary=%s" % (ntypes, binary), exact=binary)
+    for gm_args in [(0.5, 11.5, False, False, 1.0, -1.5), (0.5, 11.5, True, False, 1.0, -0.5),
+                    (0.5, 11.5, False, False, 1.3, 0.7)]:
+        rng = np.random.default_rng(11)
+        coords, tv, radii = vector_case(rng, 70, 5, 7.0)
+        ref = oracle.GridMaker(*gm_args).forward((0, 0.1, 0), coords, tv, radii)
+        got = forward_vector(gm_args, (0, 0.1, 0), coords, tv, radii)
+        close(got, ref, "vector forward %s" % (gm_args,), exact=gm_args[2])
+    # radii by type
+    rng = np.random.default_rng(12)
+    coords, tv, _ = vector_case(rng, 50, 6, 6.0)
+    tr = rng.uniform(0.8, 2.0, 6).astype(np.float32)
+    for binary in (False, True):
+        ref = oracle.GridMaker(0.5, 9.5, binary, True).forward((0, 0, 0), coords, tv, tr)
+        got = forward_vector((0.5, 9.5, binary, True), (0, 0, 0), coords, tv, tr)
+        close(got, ref, "vector forward, radii by type, binary=%s" % binary, exact=binary)
+    # a larger grid (two z slabs in the matrix-core kernel's terms): dim 60
+    rng = np.random.default_rng(13)
+    coords, tv, radii = vector_case(rng, 150, 4, 16.0)
+    ref = oracle.GridMaker(0.5, 29.5).forward((0, 0, 0), coords, tv, radii)
+    close(forward_vector((0.5, 29.5), (0, 0, 0), coords, tv, radii), ref, "vector forward dim 60")
+
+
+def group_backward_vector():
+    for binary, rti in ((False, False), (True, False), (False, True)):
+        rng = np.random.default_rng(40 + binary + 2 * rti)
+        coords, tv, radii = vector_case(rng, 40, 5, 6.0)
+        if rti:
+            radii = rng.uniform(0.8, 2.0, 5).astype(np.float32)
+        og = oracle.GridMaker(0.5, 9.5, binary, rti)
+        diff = rng.standard_normal(og.grid_shape(5)).astype(np.float32)
+        ra, rt = og.backward((0.1, 0, 0), coords, tv, radii, diff)
+        g = E.gridmaker(0.5, 9.5, binary, rti)
+        ag, tg = E.array((40, 3), fill=9.0), E.array((40, 5), fill=9.0)
+        assert lib.mg_backward_vector(ctypes.byref(g), 1, None, 40, None, E.f3((0.1, 0, 0)),
+                                      E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), 5,
+                                      E.ptr(E.put(diff)), E.ptr(ag), E.ptr(tg), None) == 0
+        _checked[0] += 1
+        assert np.allclose(ag, ra, rtol=1e-4, atol=3e-5), float(np.abs(ag - ra).max())
+        assert np.allclose(tg, rt, rtol=1e-4, atol=3e-5), float(np.abs(tg - rt).max())
+
+
+def group_second_order():
+    rng = np.random.default_rng(50)
+    coords, types, radii = synth.small_index_case(rng, 30, 3, 5.0)
+    og = oracle.GridMaker(0.5, 7.5)
+    dens = og.forward((0, 0, 0), coords, types, radii, 3)
+    diff = rng.standard_normal(dens.shape).astype(np.float32)
+    ref = og.backward_relevance((0, 0, 0), coords, types, radii, dens, diff)
+    g = E.gridmaker(0.5, 7.5)
+    rel = E.array(30, fill=9.0)
+    assert lib.mg_backward_relevance(ctypes.byref(g), 1, None, 30, None, E.f3((0, 0, 0)),
+                                     E.ptr(E.put(coords)), E.ptr(E.put(types)), E.ptr(E.put(radii)), 3,
+                                     E.ptr(E.put(dens)), E.ptr(E.put(diff)), E.ptr(rel), None) == 0
+    _checked[0] += 1
+    assert np.allclose(rel, ref, rtol=1e-4, atol=3e-5), float(np.abs(rel - ref).max())
+    coords, tv, radii = vector_case(rng, 25, 4, 5.0)
+    diff = rng.standard_normal(og.grid_shape(4)).astype(np.float32)
+    ag = rng.standard_normal((25, 3)).astype(np.float32)
+    tg = rng.standard_normal((25, 4)).astype(np.float32)
+    rdd, radd, rtdd = og.backward_gradients((0, 0, 0), coords, tv, radii, diff, ag, tg)
+    dd, add, tdd = E.array(diff.shape, fill=9.0), E.array((25, 3), fill=9.0), E.array((25, 4), fill=9.0)
+    assert lib.mg_backward_gradients(ctypes.byref(g), 1, None, 25, None, E.f3((0, 0, 0)),
+                                     E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), 4,
+                                     E.ptr(E.put(diff)), E.ptr(E.put(ag)), E.ptr(E.put(tg)), E.ptr(dd),
+                                     E.ptr(add), E.ptr(tdd), None) == 0
+    _checked[0] += 1
+    assert np.allclose(dd, rdd, rtol=1e-4, atol=3e-5), float(np.abs(dd - rdd).max())
+    assert np.allclose(add, radd, rtol=1e-4, atol=1e-4), float(np.abs(add - radd).max())
+    assert np.allclose(tdd, rtdd, rtol=1e-4, atol=3e-5), float(np.abs(tdd - rtdd).max())
+
+
+def interpolate(in_res, in_dim_a, out_res, out_dim_a, grids, quats, shifts, centers):
+    B, K = grids.shape[:2]
+    od = int(round(out_dim_a / out_res)) + 1
+    out = E.array((B, K, od, od, od), fill=9.0)
+    zeros = E.put(np.zeros((B, 3), np.float32))
+    assert lib.mg_interpolate(in_res, in_dim_a, out_res, out_dim_a, B, K, E.ptr(E.put(centers)),
+                              E.f3((0, 0, 0)), E.ptr(E.put(grids)), E.ptr(E.put(quats)),
+                              E.f4((1, 0, 0, 0)), E.ptr(zeros), E.f3((0, 0, 0)), E.ptr(E.put(shifts)),
+                              E.f3((0, 0, 0)), E.ptr(E.put(centers)), E.f3((0, 0, 0)), E.ptr(out),
+                              None) == 0
+    return out
+
+
+def group_interpolate():
+    lib.mg_interpolate_force_gather.argtypes = [ctypes.c_int]
+    rng = np.random.default_rng(60)
+    for in_res, in_a, out_res, out_a, K in [(0.5, 11.5, 0.5, 11.5, 3), (0.5, 15.5, 0.5, 15.5, 2),
+                                           (0.5, 11.5, 0.25, 5.75, 2), (0.25, 5.75, 0.5, 11.5, 2)]:
+        B = 2
+        idim = int(round(in_a / in_res)) + 1
+        grids = rng.standard_normal((B, K, idim, idim, idim)).astype(np.float32)
+        quats = synth.random_quaternions(rng, B)
+        quats[0] = (1, 0, 0, 0)
+        shifts = rng.uniform(-1.5, 1.5, (B, 3)).astype(np.float32)
+        centers = rng.uniform(-1, 1, (B, 3)).astype(np.float32)
+        ref = oracle.interpolate_batch(in_res, in_a, out_res, out_a, centers, grids, quats,
+                                       np.zeros((B, 3), np.float32), shifts, centers)
+        got = interpolate(in_res, in_a, out_res, out_a, grids, quats, shifts, centers).copy()
+        close(got, ref, "interpolate %s" % ((in_res, in_a, out_res, out_a),))
+        lib.mg_interpolate_force_gather(1)
+        gathered = interpolate(in_res, in_a, out_res, out_a, grids, quats, shifts, centers)
+        lib.mg_interpolate_force_gather(0)
+        close(gathered, got, "gather path equals staged path", exact=True)
+
+
 GROUPS = {k[len("group_"):]: v for k, v in list(globals().items()) if k.startswith("group_")}
 
 if __name__ == "__main__":
