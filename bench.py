@@ -8,7 +8,7 @@ N(0,1) upstream gradient and the un-rotation of those gradients.  All inputs are
 resident in HBM before the timed region.  One JSON line is printed.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
-                    [--no-write-stream] [--graph]
+                    [--no-write-stream] [--no-graph] [--serial-only] [--no-autotune]
 """
 import argparse
 import json
@@ -233,9 +233,13 @@ def main():
                     help="skip the forward call with every atom ignored (the write stream alone) "
                          "and the plain fill: for profiling runs, whose per-kernel means then "
                          "cover the real calls only")
-    ap.add_argument("--graph", action="store_true",
-                    help="replay the four launches of a step as one captured HIP graph (measured: "
-                         "no faster than launching them one by one, which is the default)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="do not time the step as a captured HIP graph")
+    ap.add_argument("--serial-only", action="store_true",
+                    help="time only the step in the reference's order on one stream")
+    ap.add_argument("--no-autotune", action="store_true",
+                    help="keep the library's default write-out of the splat launch instead of "
+                         "measuring both and setting the faster")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU (examples are independent; a larger job "
@@ -289,44 +293,105 @@ def main():
         gm.backward_batch(offsets, centers, moved, types, radii, diff, grads,
                           unrotate=(quats, centers))
 
-    def step():
-        # (k_backward_unrotated does the last two in one launch, bit for bit; it measures the
-        # same, see kernels.backward.unrotated_ms)
+    def step_serial():
+        # the reference's order, one stream (k_backward_unrotated does the last two in one
+        # launch, bit for bit; it measures the same, see kernels.backward.unrotated_ms)
         k_transform()
         k_forward()
         k_backward()
         k_unrotate()
 
-    run_step = step
-    if args.graph:
-        # the four launches of a step as one HIP graph: nothing in them allocates or synchronises
-        step()
-        torch.cuda.synchronize()
-        eager = (grid.clone(), grads.clone())
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        for _ in range(2):          # replays must reproduce the eager results bit for bit
-            grid.zero_()
-            grads.zero_()
-            graph.replay()
-            torch.cuda.synchronize()
-            if not (torch.equal(grid, eager[0]) and torch.equal(grads, eager[1])):
-                raise RuntimeError("HIP graph replay differs from the eager step")
-        del eager
-        run_step = graph.replay
+    side = torch.cuda.Stream()                    # default priority, like the main stream
+    ev_moved, ev_sorted = torch.cuda.Event(), torch.cuda.Event()
 
-    for _ in range(args.warmup):
-        run_step()
+    def step_overlapped():
+        # The forward and the backward pass of a step do not depend on each other, and the
+        # forward pass is two launches: the small sort launch (a chain of dependent phases that
+        # fills 40 % of the CUs for 12 us) runs on a second stream beside the backward pass
+        # instead of in front of the splat launch.  Same launches, same results.
+        main = torch.cuda.current_stream()
+        k_transform()
+        ev_moved.record(main)
+        side.wait_event(ev_moved)
+        with torch.cuda.stream(side):
+            sb = gm.sort_batch(offsets, centers, moved, types, radii, T)
+            ev_sorted.record(side)
+        k_backward()
+        main.wait_event(ev_sorted)
+        gm.splat_batch(sb, grid)
+        k_unrotate()
+
+    # which write-out the splat launch uses here: measured, the faster one is set
+    write_out = {}
+    if not args.no_autotune:
+        from libmolgrid_amd import _capi
+        for name, on in (("per_wave", 0), ("paged", 1)):
+            _capi.lib.mg_forward_index_paged(on)
+            write_out[name + "_ms"] = round(event_ms(k_forward, max(args.steps, 10)), 4)
+        use_paged = write_out["paged_ms"] < write_out["per_wave_ms"]
+        _capi.lib.mg_forward_index_paged(1 if use_paged else 0)
+        write_out["used"] = "paged" if use_paged else "per_wave"
+
+    step_serial()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step()
-    t_enqueued = time.perf_counter()              # the host has handed over every launch
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    enqueue_ms_per_step = (t_enqueued - t0) / args.steps * 1e3
+    expect = (grid.clone(), grads.clone())
+
+    def same_as_serial(what):
+        torch.cuda.synchronize()
+        if not (torch.equal(grid, expect[0]) and torch.equal(grads, expect[1])):
+            raise RuntimeError("%s differs from the serial eager step" % what)
+        grid.zero_()
+        grads.zero_()
+
+    def timed(run):
+        for _ in range(args.warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        t_enqueued = time.perf_counter()          # the host has handed over every launch
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) / args.steps * 1e3, (t_enqueued - t0) / args.steps * 1e3
+
+    # A step can be enqueued in the reference's order on one stream or with the sort beside the
+    # backward pass, and launch by launch or as one captured HIP graph (nothing in a step
+    # allocates or synchronises).  Every variant is checked against the serial eager step bit
+    # for bit and timed over exactly --steps steps; `value` is the fastest one's, all are listed.
+    variants = {}
+    order = [("serial", step_serial)]
+    if not args.serial_only:
+        order.append(("overlapped", step_overlapped))
+    for name, fn in order:
+        grid.zero_()
+        grads.zero_()
+        fn()
+        same_as_serial(name + " step")
+        variants[name + "_eager"] = timed(fn)
+        if args.no_graph:
+            continue
+        try:
+            fn()                                  # workspaces exist before the capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            for _ in range(2):                    # replays must reproduce the eager results
+                graph.replay()
+                same_as_serial("replay of the captured %s step" % name)
+            variants[name + "_graph"] = timed(graph.replay)
+        except RuntimeError as e:                 # a capture that fails is reported, not fatal
+            variants[name + "_graph"] = (float("inf"), float("inf"))
+            variants[name + "_graph_error"] = str(e)[:200]
+    del expect
+    timings = {k: v for k, v in variants.items() if isinstance(v, tuple)}
+    best = min(timings, key=lambda k: timings[k][0])
+    ms_per_step, enqueue_ms_per_step = timings[best]
+    step_variants = {k: ({"ms_per_step": round(v[0], 4), "enqueue_ms_per_step": round(v[1], 4)}
+                         if isinstance(v, tuple) else v) for k, v in variants.items()}
+    step = step_serial
+    step()                                        # the grids and gradients of a step again
 
     # per-kernel durations (events on the launch stream)
     it = max(args.steps, 10)
@@ -454,11 +519,13 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "launch": "hip graph replay" if args.graph else "eager",
+        "launch": best,
         "ms_per_step": round(ms_per_step, 4),
         # wall time the host needs to enqueue a step (the timed loop before its synchronize): when
         # this comes close to ms_per_step the loop is bound by the host, not by the kernels
         "enqueue_ms_per_step": round(enqueue_ms_per_step, 4),
+        "step_variants": step_variants,
+        "forward_write_out": write_out or None,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

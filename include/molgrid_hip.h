@@ -119,6 +119,25 @@ int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
                         const float* type_index, const float* radii, int ntypes, float* out,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* The two launches of mg_forward_index_ws as calls of their own, for callers that
+ * want the sort off the critical path (enqueued on another stream beside other
+ * work, e.g. the backward pass of the previous batch): mg_forward_index_sort
+ * reads the atoms and fills `workspace`; mg_forward_index_splat reads only the
+ * workspace and writes `out`.  Both must be given the same g, nbatch,
+ * atoms_per_example, ntypes and workspace size, and the splat must be ordered
+ * after the sort (same stream, or an event).  The grids are those of
+ * mg_forward_index_ws, bit for bit.  No counterpart in the reference, whose
+ * forward_gpu scans the atoms inside the gridding kernel
+ * (src/grid_maker.cu:176-210). */
+int mg_forward_index_sort(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_index, const float* radii, int ntypes,
+                          void* workspace, size_t workspace_bytes, void* stream);
+int mg_forward_index_splat(const mg_gridmaker* g, int nbatch, int atoms_per_example, int ntypes,
+                           float* out, const void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* Host only.  Bytes of workspace mg_forward_index_ws needs for these sizes (0
  * for an empty call). */
 size_t mg_forward_index_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,

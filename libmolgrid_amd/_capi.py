@@ -19,7 +19,8 @@ MG_STATIC_SCRATCH_BYTES = 16 << 20
 EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
-    "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_index_paged", "mg_forward_vector", "mg_backward_index",
+    "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_index_paged",
+    "mg_forward_index_sort", "mg_forward_index_splat", "mg_forward_vector", "mg_backward_index",
     "mg_backward_index_unrotated",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate", "mg_interpolate_force_gather",
     "mg_narrow", "mg_widen",
@@ -73,6 +74,8 @@ def declare(lib):
     lib.mg_forward_index.argtypes = fwd
     lib.mg_forward_index_static.argtypes = fwd
     lib.mg_forward_index_ws.argtypes = fwd[:-1] + [_vp, ctypes.c_size_t, _vp]
+    lib.mg_forward_index_sort.argtypes = fwd[:-2] + [_vp, ctypes.c_size_t, _vp]
+    lib.mg_forward_index_splat.argtypes = [gm, _i, _i, _i, _vp, _vp, ctypes.c_size_t, _vp]
     lib.mg_forward_index_workspace_size.argtypes = [gm, _i, _i, _i]
     lib.mg_forward_index_workspace_size.restype = ctypes.c_size_t
     lib.mg_forward_vector.argtypes = fwd

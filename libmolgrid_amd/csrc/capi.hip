@@ -238,6 +238,48 @@ int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
                             workspace_bytes, stream);
 }
 
+int mg_forward_index_sort(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                          int atoms_per_example, const float* grid_centers,
+                          const float grid_center_host[3], const float* coords,
+                          const float* type_index, const float* radii, int ntypes,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  bool nothing = false;
+  const float* const no_grid = reinterpret_cast<const float*>(16);    // only tested against NULL
+  const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
+                                    radii, ntypes, no_grid, &nothing);
+  if (s != MG_OK || nothing) return s;
+  if (workspace == nullptr) return MG_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return MG_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes))
+    return MG_ERR_INVALID_ARGUMENT;
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
+  const hipError_t e = launch_sort_atoms(grid_arg(g, ntypes), batch, nbatch,
+                                         vec3(grid_centers, grid_center_host), coords, type_index,
+                                         radii, g->binary != 0, workspace, workspace_bytes,
+                                         (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return MG_ERR_UNSUPPORTED;
+  return from_hip(e);
+}
+
+int mg_forward_index_splat(const mg_gridmaker* g, int nbatch, int atoms_per_example, int ntypes,
+                           float* out, const void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  int s = check_common(g, nbatch, nullptr, atoms_per_example, ntypes);
+  if (s != MG_OK) return s;
+  if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || ntypes == 0) return MG_OK;
+  if (out == nullptr || workspace == nullptr) return MG_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return MG_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes))
+    return MG_ERR_INVALID_ARGUMENT;
+  const hipError_t e = launch_splat_sorted(grid_arg(g, ntypes), nbatch, atoms_per_example, out,
+                                           g->binary != 0, needs_exact(g),
+                                           const_cast<void*>(workspace), workspace_bytes,
+                                           (hipStream_t)stream);
+  if (e == hipErrorInvalidValue) return MG_ERR_UNSUPPORTED;
+  return from_hip(e);
+}
+
 int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                      int atoms_per_example, const float* grid_centers,
                      const float grid_center_host[3], const float* coords,

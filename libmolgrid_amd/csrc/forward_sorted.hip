@@ -766,32 +766,55 @@ size_t forward_sorted_workspace_bytes(int nbatch, int atoms_per_example, int nty
          (size_t)capacity * 16;
 }
 
+namespace {
+
 // hipErrorInvalidValue = the case is not covered (a channel of 4 GB or more, more records than a
 // buffer addresses, a workspace that is too small).
-hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nbatch,
-                                 const Vec3Arg& centers, const float* coords,
-                                 const float* type_index, const float* radii, float* out,
-                                 bool binary, bool exact, void* workspace, size_t workspace_bytes,
-                                 hipStream_t stream) {
+hipError_t sorted_layout(const GridArg& g, int nbatch, int per_example, void* workspace,
+                         size_t workspace_bytes, SortedAtoms* s, int* nxs_out) {
   const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
   if (chan_stride * 4 >= 0xfffffff0ull) return hipErrorInvalidValue;
-  const long long capacity = (long long)nbatch * batch.per_example;
+  const long long capacity = (long long)nbatch * per_example;
   if (capacity * 16 >= 0xfffffff0ll) return hipErrorInvalidValue;
   if (workspace == nullptr ||
-      workspace_bytes < forward_sorted_workspace_bytes(nbatch, batch.per_example, g.ntypes, g.dim))
+      workspace_bytes < forward_sorted_workspace_bytes(nbatch, per_example, g.ntypes, g.dim))
     return hipErrorInvalidValue;
   const int nxs = (g.dim + kColXY - 1) / kColXY;
   if ((long long)g.ntypes * nxs >= (1 << 26)) return hipErrorInvalidValue;
-  const SortedAtoms s = carve(workspace, nbatch, g.ntypes * nxs, capacity);
+  *s = carve(workspace, nbatch, g.ntypes * nxs, capacity);
+  *nxs_out = nxs;
+  return hipSuccess;
+}
+
+}  // namespace
+
+// First launch of the forward pass: the atoms -> sorted records and tables in the workspace.
+hipError_t launch_sort_atoms(const GridArg& g, const BatchArg& batch, int nbatch,
+                             const Vec3Arg& centers, const float* coords, const float* type_index,
+                             const float* radii, bool binary, void* workspace,
+                             size_t workspace_bytes, hipStream_t stream) {
+  SortedAtoms s;
+  int nxs = 0;
+  const hipError_t e = sorted_layout(g, nbatch, batch.per_example, workspace, workspace_bytes, &s, &nxs);
+  if (e != hipSuccess) return e;
   // channels per workgroup of the sort: a few, and no more keys than it handles
   const int per_part = std::max(1, std::min(kSortChannels, kKeyGroup / nxs));
   const int parts = (g.ntypes + per_part - 1) / per_part;
   hipLaunchKernelGGL(sort_atoms_kernel, dim3((unsigned)(parts * nbatch)), dim3(kSortThreads), 0, stream, g,
                      batch, nbatch, nxs, parts, per_part, binary ? 1.0f : g.frm, centers, coords,
                      type_index, radii, s.slot_info, s.cand, s.records, s.capacity);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
+  return hipGetLastError();
+}
 
+// Second launch: the workspace that launch_sort_atoms filled for the same sizes and the same
+// density mode -> the grids.
+hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_example, float* out,
+                               bool binary, bool exact, void* workspace, size_t workspace_bytes,
+                               hipStream_t stream) {
+  SortedAtoms s;
+  int nxs = 0;
+  const hipError_t e = sorted_layout(g, nbatch, atoms_per_example, workspace, workspace_bytes, &s, &nxs);
+  if (e != hipSuccess) return e;
   if (exact) {
     if (binary) return launch_splat<true, true, 1>(g, s, nbatch, out, stream);
     return launch_splat<false, true, 1>(g, s, nbatch, out, stream);
@@ -802,6 +825,18 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
   }
   if (binary) return launch_splat<true, false, 2>(g, s, nbatch, out, stream);
   return launch_splat<false, false, 2>(g, s, nbatch, out, stream);
+}
+
+hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nbatch,
+                                 const Vec3Arg& centers, const float* coords,
+                                 const float* type_index, const float* radii, float* out,
+                                 bool binary, bool exact, void* workspace, size_t workspace_bytes,
+                                 hipStream_t stream) {
+  const hipError_t e = launch_sort_atoms(g, batch, nbatch, centers, coords, type_index, radii, binary,
+                                         workspace, workspace_bytes, stream);
+  if (e != hipSuccess) return e;
+  return launch_splat_sorted(g, nbatch, batch.per_example, out, binary, exact, workspace,
+                             workspace_bytes, stream);
 }
 
 int set_forward_paged(int on) { return g_paged.exchange(on ? 1 : 0); }

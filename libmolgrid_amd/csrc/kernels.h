@@ -37,6 +37,17 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
                                  bool binary, bool exact, void* workspace, size_t workspace_bytes,
                                  hipStream_t stream);
 
+// The two launches of launch_forward_sorted on their own, for callers that enqueue them apart
+// (the sort on another stream, beside other work): the splat launch needs the workspace the sort
+// launch filled for the same nbatch, atoms_per_example, ntypes, grid and density mode.
+hipError_t launch_sort_atoms(const GridArg& g, const BatchArg& batch, int nbatch,
+                             const Vec3Arg& centers, const float* coords, const float* type_index,
+                             const float* radii, bool binary, void* workspace,
+                             size_t workspace_bytes, hipStream_t stream);
+hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_example, float* out,
+                               bool binary, bool exact, void* workspace, size_t workspace_bytes,
+                               hipStream_t stream);
+
 // Which write-out the splat launch uses for grids of up to 48 voxels a side with rows of whole
 // float4 pieces: 1 = workgroups that own a slab of four x planes of one channel and write it as
 // whole 4 KB pages, 0 = one wave per territory writing its own rows.  Same grids bit for bit.

@@ -327,6 +327,15 @@ class AtomBatch(object):
         return self._dev
 
 
+class SortedBatch(object):
+    """What ``GridMaker.sort_batch`` leaves for ``GridMaker.splat_batch``: the device workspace
+    with the sorted atom records and their tables, and the sizes it was made for."""
+
+    def __init__(self, workspace, nbytes, nbatch, largest, ntypes):
+        self.workspace, self.nbytes = workspace, nbytes
+        self.nbatch, self.largest, self.ntypes = nbatch, largest, ntypes
+
+
 def _offsets_arg(offsets):
     """(device int32 tensor, nbatch, largest example, total atoms) for a ragged batch."""
     b = offsets if isinstance(offsets, AtomBatch) else AtomBatch(offsets)
@@ -1336,6 +1345,51 @@ class GridMaker(object):
         code = fn(self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3), a_coords.ptr,
                   a_types.ptr, a_radii.ptr, T, a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward_batch")
+        a_out.finish()
+
+    @_accepts_grids
+    def sort_batch(self, offsets, centers, coords, types, radii, ntypes):
+        """First half of ``forward_batch`` for index types: sorts the atoms of a ragged batch
+        into a device workspace and returns it as a ``SortedBatch``; ``splat_batch`` turns it
+        into grids.  The two halves may be enqueued on different streams (the caller orders the
+        splat after the sort, e.g. with an event), which takes the sort launch off the critical
+        path when other work -- the backward pass -- can run beside it.  The grids are those of
+        ``forward_batch`` bit for bit."""
+        off, B, largest, total = _offsets_arg(offsets)
+        cen = _small_device(centers, 3)
+        a_coords, a_types, a_radii = _Arg(coords, "coords", 2), _Arg(types, "types", 1), \
+            _Arg(radii, "radii", 1)
+        if self._p.radii_type_indexed:
+            raise ValueError("Type indexed radii not supported with index types.")
+        if cen.shape[0] != B:
+            raise ValueError("Mismatched batch sizes: %d vs %d" % (cen.shape[0], B))
+        if a_coords.shape[0] < total or a_types.shape[0] < total or a_radii.shape[0] < total:
+            raise IndexError("atom arrays are shorter than offsets[-1]")
+        T = int(ntypes)
+        self._check_host_types(types, T)
+        need = int(_lib.mg_forward_index_workspace_size(self._p, B, largest, T))
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=_device())
+        code = _lib.mg_forward_index_sort(self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3),
+                                          a_coords.ptr, a_types.ptr, a_radii.ptr, T,
+                                          ws.data_ptr(), need, _stream())
+        _capi.check(code, "GridMaker.sort_batch")
+        return SortedBatch(ws, need, B, largest, T)
+
+    @_accepts_grids
+    def splat_batch(self, sorted_batch, grid):
+        """Second half of ``forward_batch``: the grids (B,T,D,D,D) of a ``SortedBatch``."""
+        a_out = _Arg(grid, "grid", 5, out=True, wide=True)
+        sb = sorted_batch
+        if a_out.shape[0] != sb.nbatch or a_out.shape[1] != sb.ntypes:
+            raise ValueError("grid is %s but the atoms were sorted for %d examples and %d types"
+                             % (a_out.shape, sb.nbatch, sb.ntypes))
+        self._check_grid(a_out.shape[1:])
+        # the workspace may have been allocated under another stream: tell the allocator that
+        # this stream uses it too
+        sb.workspace.record_stream(torch.cuda.current_stream())
+        code = _lib.mg_forward_index_splat(self._p, sb.nbatch, sb.largest, sb.ntypes, a_out.ptr,
+                                           sb.workspace.data_ptr(), sb.nbytes, _stream())
+        _capi.check(code, "GridMaker.splat_batch")
         a_out.finish()
 
     # -- backward -----------------------------------------------------------

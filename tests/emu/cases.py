@@ -172,6 +172,34 @@ def group_forward_batch():
     _checked[0] += 1
 
 
+def group_forward_split():
+    """mg_forward_index_sort + mg_forward_index_splat give the grids of mg_forward_index_ws."""
+    cfg = synth.index_batch(2, 5, (30, 120), (3, 9), ntypes=6)
+    off = cfg["offsets"]
+    width = int(np.diff(off).max())
+    for binary in (False, True):
+        g = E.gridmaker(0.5, 11.5, binary)
+        dim = int(g.dim)
+        whole = forward_index((0.5, 11.5, binary), cfg["centers"], cfg["coords"], cfg["types"],
+                              cfg["radii"], 6, offsets=off, per_example=width, nbatch=5)
+        need = lib.mg_forward_index_workspace_size(ctypes.byref(g), 5, width, 6)
+        ws = E.array(need, np.uint8, tight=False)
+        out = E.array((5, 6, dim, dim, dim), fill=7.0)
+        assert lib.mg_forward_index_sort(ctypes.byref(g), 5, E.ptr(E.put(off, np.int32)), width,
+                                         E.ptr(E.put(cfg["centers"])), E.f3((0, 0, 0)),
+                                         E.ptr(E.put(cfg["coords"])), E.ptr(E.put(cfg["types"])),
+                                         E.ptr(E.put(cfg["radii"])), 6, E.ptr(ws), need, None) == 0
+        assert np.all(out == 7.0)                       # the sort does not touch the grids
+        assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(ws), need,
+                                          None) == 0
+        close(out, whole, "sort + splat, binary=%s" % binary, exact=True)
+    # argument errors: a workspace that is too small or misaligned, no workspace
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(ws), need - 1, None) == -1
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), ws[16:].ctypes.data, need, None) == -1
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), None, need, None) == -4
+    _checked[0] += 1
+
+
 def group_forward_paged():
     """The paged write-out (workgroups that own a slab and write whole 4 KB pages) gives the grids
     of the per-wave write-out bit for bit: dims 16, 24, 48 and smaller, binary and Gaussian, batches

@@ -24,7 +24,7 @@ def emulated_library():
     return build_emu.build()
 
 
-@pytest.mark.parametrize("group", ["transform", "forward_index", "forward_batch", "forward_paged", "backward_index",
+@pytest.mark.parametrize("group", ["transform", "forward_index", "forward_batch", "forward_paged", "forward_split", "backward_index",
                                    "forward_vector", "backward_vector", "second_order", "interpolate"])
 def test_group(emulated_library, group):
     p = subprocess.run([sys.executable, RUNNER, group], stdout=subprocess.PIPE,
