@@ -67,20 +67,6 @@ constexpr int kRawBufferFlags = 0x00020000;   // untyped 32-bit elements, no swi
 // a * b with 0 * anything = 0 (also infinities and NaNs)
 __device__ __forceinline__ float mul_zero_wins(float a, float b) { return mul_legacy(a, b); }
 
-// Voxel range [lo, lo + n) along one axis whose centres lie within `reach` of `coord` (n <= 0:
-// none).  Tighter than the reference's index box (src/grid_maker.cu:66-79), which adds a voxel
-// beyond the reach on either side; such voxels contribute nothing to a gradient.  The slack keeps
-// every voxel that rounding could put on the inner side of the cut-off: whether it counts is
-// decided by the distance test of the voxel itself.
-__device__ __forceinline__ void reach_range(float origin, float coord, float reach, float inv_res,
-                                            int dim, int& lo, int& n) {
-  constexpr float kSlack = 1e-3f;
-  const float first = fmaxf(ceilf((coord - reach - origin) * inv_res - kSlack), 0.f);
-  const float last = fminf(floorf((coord + reach - origin) * inv_res + kSlack), (float)(dim - 1));
-  lo = (int)first;
-  n = (int)last - lo + 1;
-}
-
 // Atom gradients for index types.  One wave per atom.  The (y, z) columns of the atom's box that
 // come within reach of the atom are compacted into a wave-private list (a circle's worth of
 // columns instead of the square's), each lane takes one column of the list and marches along x;
@@ -270,6 +256,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
     const float* __restrict__ type_vector, const float* __restrict__ radii,
     const float* __restrict__ diff, float* __restrict__ atom_gradients,
     float* __restrict__ type_gradients) {
+  __shared__ int s_cols[kBwdWaves][2 * kWave];   // column list of each wave (sweep_reach)
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: so is the atom
   const int b = blockIdx.y;
@@ -303,12 +290,10 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
       }
       const GradConsts gc = grad_consts(g, ar);
       const float inv_ar2 = gc.inv_ar2;
-      int lo0, hi0, lo1, hi1, lo2, hi2;
-      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
-      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
-      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
-      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
-      const bool any = ni > 0 && nj > 0 && nk > 0 && ar > 0.f;   // no extent: no gradient
+      const bool any = ar > 0.f && densityrad > 0.f;             // no extent: no gradient
+      // density and gradient scale vanish beyond the final radius; a binary sphere wider than
+      // its index box is cut by the box
+      const bool index_box = BINARY && g.frm < 1.0f;
       for (int cbase = 0; cbase < T; cbase += TG) {
         const int nchan = min(TG, T - cbase);
         float tg[TG];
@@ -316,7 +301,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         for (int t = 0; t < TG; ++t) tg[t] = 0.f;
         if (any) {
           const float* group = diff_b + (size_t)cbase * chan_stride;
-          sweep_box(g, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
+          sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad, index_box,
                     [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
                         unsigned lane_off, bool live) {
                       float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
@@ -359,16 +344,14 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         }
         const GradConsts gc = grad_consts(g, ar);
         const float inv_ar2 = gc.inv_ar2;
-        int lo0, hi0, lo1, hi1, lo2, hi2;
-        bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
-        bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
-        bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
-        const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
         float tgt = 0.f, tx = 0.f, ty = 0.f, tz = 0.f;
-        if (ni > 0 && nj > 0 && nk > 0 && ar > 0.f) {
+        if (ar > 0.f && densityrad > 0.f) {
           const float* chan = diff_b + (size_t)t * chan_stride;
-          sweep_channel(g, chan, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
-                        [&](float dx, float dy, float dz, float dist2, float gv, bool live) {
+          sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
+                      BINARY && g.frm < 1.0f,
+                        [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
+                            unsigned lane_off, bool live) {
+                          const float gv = (chan + plane_off)[lane_off];
                           float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
                           if (!live) val = 0.f;
                           tgt = fmaf(val, gv, tgt);

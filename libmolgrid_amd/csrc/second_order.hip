@@ -55,6 +55,7 @@ __global__ __launch_bounds__(kThreads) void relevance_kernel(
     const float* __restrict__ type_index, const float* __restrict__ radii,
     const float* __restrict__ density_grid, const float* __restrict__ diff,
     float* __restrict__ relevance) {
+  __shared__ int s_cols[kWaves][2 * kWave];      // column list of each wave (sweep_reach)
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = blockIdx.y;
@@ -80,22 +81,19 @@ __global__ __launch_bounds__(kThreads) void relevance_kernel(
         densityrad = radius * g.radius_scale * g.frm;
         ar = radius * g.radius_scale;
       }
-      int lo0, hi0, lo1, hi1, lo2, hi2;
-      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
-      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
-      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
-      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
-      if (ni > 0 && nj > 0 && nk > 0) {
+      // the voxels with a density above zero lie within the final radius (binary: the radius)
+      if (densityrad > 0.f) {
         const float* dens = density_grid + example + (size_t)(int)tf * chan_stride;
         const float* dif = diff + example + (size_t)(int)tf * chan_stride;
-        sweep_box(g, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
-                  [&](float dx, float dy, float dz, float, unsigned plane_off, unsigned lane_off,
-                      bool live) {
-                    const float val = calc_point_reference<BINARY>(g, dx, dy, dz, ar);
-                    const float denseval = (dens + plane_off)[lane_off];
-                    const float gridval = (dif + plane_off)[lane_off];
-                    if (live && val > 0.f && denseval > 0.f) ret += gridval * val / denseval;
-                  });
+        sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
+                    BINARY && g.frm < 1.0f,
+                    [&](float dx, float dy, float dz, float, unsigned plane_off, unsigned lane_off,
+                        bool live) {
+                      const float val = calc_point_reference<BINARY>(g, dx, dy, dz, ar);
+                      const float denseval = (dens + plane_off)[lane_off];
+                      const float gridval = (dif + plane_off)[lane_off];
+                      if (live && val > 0.f && denseval > 0.f) ret += gridval * val / denseval;
+                    });
       }
     }
     ret = wave_sum(ret);
@@ -116,6 +114,7 @@ __global__ __launch_bounds__(kThreads) void grad_grad_kernel(
     const float* __restrict__ diff, const float* __restrict__ atom_gradients,
     const float* __restrict__ type_gradients, float* __restrict__ diffdiff,
     float* __restrict__ atom_diffdiff, float* __restrict__ type_diffdiff) {
+  __shared__ int s_cols[kWaves][2 * kWave];      // column list of each wave (sweep_reach)
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = blockIdx.y;
@@ -149,17 +148,12 @@ __global__ __launch_bounds__(kThreads) void grad_grad_kernel(
         densityrad = radius * g.radius_scale * g.frm;
         ar = radius * g.radius_scale;
       }
-      int lo0, hi0, lo1, hi1, lo2, hi2;
-      bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
-      bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
-      bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
-      const int ni = hi0 - lo0, nj = hi1 - lo1, nk = hi2 - lo2;
-      if (ni <= 0 || nj <= 0 || nk <= 0) continue;
+      if (!(densityrad > 0.f)) continue;
       const float inv_ar = 1.0f / ar, inv_ar2 = inv_ar * inv_ar;
       const float rcut = ar * g.frm, rcore = ar * g.grm;
       const float* dif = diff + example + (size_t)t * chan_stride;
       float* dd = diffdiff + example + (size_t)t * chan_stride;
-      sweep_box(g, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, ni, nj, nk,
+      sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
                 [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
                     unsigned lane_off, bool live) {
                   const float dist = sqrtf(dist2);

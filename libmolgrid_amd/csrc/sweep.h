@@ -116,6 +116,104 @@ __device__ __forceinline__ void sweep_channel(const GridArg& g, const float* __r
   }
 }
 
+// Voxel range [lo, lo + n) along one axis whose centres lie within `reach` of `coord` (n <= 0:
+// none).  Tighter than the reference's index box (src/grid_maker.cu:66-79), which adds a voxel
+// beyond the reach on either side; such voxels contribute nothing to a gradient.  The slack keeps
+// a voxel whose distance equals the reach to rounding.
+__device__ __forceinline__ void reach_range(float origin, float coord, float reach, float inv_res,
+                                            int dim, int& lo, int& n) {
+  constexpr float kSlack = 1e-3f;
+  const float first = fmaxf(ceilf((coord - reach - origin) * inv_res - kSlack), 0.f);
+  const float last = fminf(floorf((coord + reach - origin) * inv_res + kSlack), (float)(dim - 1));
+  lo = (int)first;
+  n = (int)last - lo + 1;
+}
+
+// Sweep of the voxels within `reach` of an atom by one wave: like sweep_box, but over the range
+// of reach_range instead of the reference's index box, and only over the (y, z) columns that come
+// within reach of the atom -- a circle's worth instead of the square's.  The columns are tested
+// 64 at a time and compacted into `cols`, a list of 2 * kWave ints in LDS that belongs to the
+// calling wave alone; every full 64 (and the rest at the end) is marched along x, one column per
+// lane.  The set of voxels visited is a superset (by a relative slack of 1e-5 on reach^2 and
+// 1e-3 voxel on the range) of those with dist <= reach, so a body that adds nothing beyond the
+// reach gives the sums of sweep_box over the index box, in another order.
+// body(dx, dy, dz, dist2, plane_off, lane_off, live) as for sweep_box.
+template <typename Body>
+__device__ __forceinline__ void sweep_reach(const GridArg& g, int lane, volatile int* cols,
+                                            float ox, float oy, float oz, float ax, float ay,
+                                            float az, float reach, Body body) {
+  const int dim = g.dim;
+  const float inv_res = 1.0f / g.resolution;
+  int lo0, lo1, lo2, ni, nj, nk;
+  reach_range(ox, ax, reach, inv_res, dim, lo0, ni);
+  reach_range(oy, ay, reach, inv_res, dim, lo1, nj);
+  reach_range(oz, az, reach, inv_res, dim, lo2, nk);
+  if (ni <= 0 || nj <= 0 || nk <= 0) return;
+  const float reach2 = reach * reach * 1.00001f;
+  const int ncols = nj * nk;
+  const float inv_nk = __builtin_amdgcn_rcpf((float)nk);
+  for (int i0 = 0; i0 < ni; i0 += kWave) {
+    const int planes = min(kWave, ni - i0);
+    const int dx_lane = __float_as_int(grid_coord(ox, lo0 + i0 + lane, g.resolution) - ax);
+    // one pass: lanes below `count` take the columns cols[0 .. count)
+    auto march = [&](int count) {
+      wave_lds_fence();                          // the list is complete
+      const bool live = lane < count;
+      const int packed = cols[live ? lane : 0];
+      const int j = packed >> 16, k = packed & 0xffff;
+      const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+      const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+      const float dyz2 = live ? dy * dy + dz * dz : INFINITY;
+      const unsigned lane_off = (unsigned)((lo1 + j) * dim + lo2 + k);
+      // (unrolled so that the loads of a few planes are in flight together)
+#pragma unroll 4
+      for (int i = 0; i < planes; ++i) {
+        const float dx = __int_as_float(__builtin_amdgcn_readlane(dx_lane, i));
+        const unsigned plane_off = (unsigned)(lo0 + i0 + i) * (unsigned)(dim * dim);
+        body(dx, dy, dz, fmaf(dx, dx, dyz2), plane_off, lane_off, live);
+      }
+    };
+    int pending = 0;
+    for (int c0 = 0; c0 < ncols; c0 += kWave) {
+      wave_lds_fence();                          // the entries moved to the front have been read
+      const int cand = c0 + lane;
+      const int j = (int)(((float)cand + 0.5f) * inv_nk), k = cand - j * nk;
+      const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
+      const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
+      const bool within = cand < ncols && dy * dy + dz * dz <= reach2;
+      const unsigned long long m = __ballot(within);
+      if (within) cols[pending + __popcll(m & ((1ull << lane) - 1ull))] = (j << 16) | k;
+      pending += __popcll(m);
+      if (pending >= kWave) {
+        march(kWave);
+        pending -= kWave;
+        const int moved = cols[kWave + lane];
+        if (lane < pending) cols[lane] = moved;
+      }
+    }
+    if (pending > 0) march(pending);
+  }
+}
+
+// sweep_reach, or -- `index_box` -- the reference's index box for the radius `reach` (sweep_box): for
+// the one case in which that box is SMALLER than the support of the density, a binary sphere with
+// a final radius multiple below one, where the box decides which voxels count.
+template <typename Body>
+__device__ __forceinline__ void sweep_reach(const GridArg& g, int lane, volatile int* cols,
+                                            float ox, float oy, float oz, float ax, float ay,
+                                            float az, float reach, bool index_box, Body body) {
+  if (index_box) {
+    int lo0, hi0, lo1, hi1, lo2, hi2;
+    bounds_1d(ox, ax, reach, g.resolution, g.dim, lo0, hi0);
+    bounds_1d(oy, ay, reach, g.resolution, g.dim, lo1, hi1);
+    bounds_1d(oz, az, reach, g.resolution, g.dim, lo2, hi2);
+    if (hi0 > lo0 && hi1 > lo1 && hi2 > lo2)
+      sweep_box(g, lane, ox, oy, oz, ax, ay, az, lo0, lo1, lo2, hi0 - lo0, hi1 - lo1, hi2 - lo2, body);
+    return;
+  }
+  sweep_reach(g, lane, cols, ox, oy, oz, ax, ay, az, reach, body);
+}
+
 }  // namespace mg
 
 #endif

@@ -361,52 +361,96 @@ def group_forward_vector():
 
 
 def group_backward_vector():
-    for binary, rti in ((False, False), (True, False), (False, True)):
-        rng = np.random.default_rng(40 + binary + 2 * rti)
-        coords, tv, radii = vector_case(rng, 40, 5, 6.0)
+    """The cases and bounds of tests/test_vector_gpu.py::test_backward_vs_oracle, plus a binary
+    sphere that is wider than its index box (final radius multiple below one)."""
+    cases = [(3, (0.5, 9.5, False, False)), (28, (0.5, 9.5, False, False)), (37, (0.5, 9.5, False, False)),
+             (5, (0.5, 9.5, True, False)), (6, (0.5, 9.5, False, True)), (6, (0.5, 9.5, True, True)),
+             (4, (0.5, 9.5, True, False, 1.0, -0.5)), (4, (0.5, 9.5, False, False, 1.3, 0.7))]
+    for ntypes, gm_args in cases:
+        rti = gm_args[3]
+        rng = np.random.default_rng(300 + ntypes)
+        coords, tv, radii = vector_case(rng, 40, ntypes, 6.0)
         if rti:
-            radii = rng.uniform(0.8, 2.0, 5).astype(np.float32)
-        og = oracle.GridMaker(0.5, 9.5, binary, rti)
-        diff = rng.standard_normal(og.grid_shape(5)).astype(np.float32)
-        ra, rt = og.backward((0.1, 0, 0), coords, tv, radii, diff)
-        g = E.gridmaker(0.5, 9.5, binary, rti)
-        ag, tg = E.array((40, 3), fill=9.0), E.array((40, 5), fill=9.0)
-        assert lib.mg_backward_vector(ctypes.byref(g), 1, None, 40, None, E.f3((0.1, 0, 0)),
-                                      E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), 5,
-                                      E.ptr(E.put(diff)), E.ptr(ag), E.ptr(tg), None) == 0
+            radii = rng.uniform(0.8, 2.0, ntypes).astype(np.float32)
+        og = oracle.GridMaker(*gm_args)
+        diff = rng.standard_normal(og.grid_shape(ntypes)).astype(np.float32)
+        ra32, rt32 = og.backward((0, 0, 0), coords, tv, radii, diff)
+        ra64, rt64 = og.backward((0, 0, 0), coords, tv, radii, diff, f64=True)
+        ma, mt = og.backward((0, 0, 0), coords, np.abs(tv), radii, np.abs(diff), f64=True)
+        ma = np.abs(ma).max(axis=1, keepdims=True) + 1e-30
+        g = E.gridmaker(*gm_args)
+        ag, tg = E.array((40, 3), fill=9.0), E.array((40, ntypes), fill=9.0)
+        assert lib.mg_backward_vector(ctypes.byref(g), 1, None, 40, None, E.f3((0, 0, 0)),
+                                      E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)),
+                                      ntypes, E.ptr(E.put(diff)), E.ptr(ag), E.ptr(tg), None) == 0
         _checked[0] += 1
-        assert np.allclose(ag, ra, rtol=1e-4, atol=3e-5), float(np.abs(ag - ra).max())
-        assert np.allclose(tg, rt, rtol=1e-4, atol=3e-5), float(np.abs(tg - rt).max())
+        a64, t64 = np.asarray(ag, np.float64), np.asarray(tg, np.float64)
+        what = "vector backward T=%d %s" % (ntypes, gm_args)
+        assert (np.abs(a64 - ra64) <= ATOL + RTOL * np.abs(ra64) + 16 * EPS * ma).all(), what
+        assert (np.abs(a64 - ra32) <= ATOL + RTOL * np.abs(ra32) + 64 * EPS * ma).all(), what
+        assert (np.abs(t64 - rt64) <= ATOL + RTOL * np.abs(rt64) + 16 * EPS * mt).all(), what
+        assert (np.abs(t64 - rt32) <= ATOL + RTOL * np.abs(rt32) + 64 * EPS * mt).all(), what
+
+
+def close_sums(got, ref, scale, what):
+    """|got - ref| <= 1e-6 + 1e-5 |ref| + 64 eps * (sum of |terms|), as tests/test_second_order_gpu.py"""
+    _checked[0] += 1
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    tol = 1e-6 + 1e-5 * np.abs(ref) + 64 * EPS * np.asarray(scale, np.float64)
+    bad = np.abs(got - ref) > tol
+    assert not bad.any(), "%s: %d values off, worst %g" % (what, int(bad.sum()), np.abs(got - ref)[bad].max())
 
 
 def group_second_order():
-    rng = np.random.default_rng(50)
-    coords, types, radii = synth.small_index_case(rng, 30, 3, 5.0)
-    og = oracle.GridMaker(0.5, 7.5)
-    dens = og.forward((0, 0, 0), coords, types, radii, 3)
-    diff = rng.standard_normal(dens.shape).astype(np.float32)
-    ref = og.backward_relevance((0, 0, 0), coords, types, radii, dens, diff)
-    g = E.gridmaker(0.5, 7.5)
-    rel = E.array(30, fill=9.0)
-    assert lib.mg_backward_relevance(ctypes.byref(g), 1, None, 30, None, E.f3((0, 0, 0)),
-                                     E.ptr(E.put(coords)), E.ptr(E.put(types)), E.ptr(E.put(radii)), 3,
-                                     E.ptr(E.put(dens)), E.ptr(E.put(diff)), E.ptr(rel), None) == 0
-    _checked[0] += 1
-    assert np.allclose(rel, ref, rtol=1e-4, atol=3e-5), float(np.abs(rel - ref).max())
-    coords, tv, radii = vector_case(rng, 25, 4, 5.0)
-    diff = rng.standard_normal(og.grid_shape(4)).astype(np.float32)
-    ag = rng.standard_normal((25, 3)).astype(np.float32)
-    tg = rng.standard_normal((25, 4)).astype(np.float32)
-    rdd, radd, rtdd = og.backward_gradients((0, 0, 0), coords, tv, radii, diff, ag, tg)
-    dd, add, tdd = E.array(diff.shape, fill=9.0), E.array((25, 3), fill=9.0), E.array((25, 4), fill=9.0)
-    assert lib.mg_backward_gradients(ctypes.byref(g), 1, None, 25, None, E.f3((0, 0, 0)),
-                                     E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), 4,
-                                     E.ptr(E.put(diff)), E.ptr(E.put(ag)), E.ptr(E.put(tg)), E.ptr(dd),
-                                     E.ptr(add), E.ptr(tdd), None) == 0
-    _checked[0] += 1
-    assert np.allclose(dd, rdd, rtol=1e-4, atol=3e-5), float(np.abs(dd - rdd).max())
-    assert np.allclose(add, radd, rtol=1e-4, atol=1e-4), float(np.abs(add - radd).max())
-    assert np.allclose(tdd, rtdd, rtol=1e-4, atol=3e-5), float(np.abs(tdd - rtdd).max())
+    """The cases of tests/test_second_order_gpu.py on the CPU."""
+    for gm_args in ((0.5, 11.5, False), (0.5, 11.5, True), (0.5, 11.5, True, False, 1.0, -0.5)):
+        binary = gm_args[2]
+        rng = np.random.default_rng(31)
+        n, T = 90, 5
+        coords = rng.uniform(-6, 6, (n, 3)).astype(np.float32)
+        types = rng.integers(0, T, n).astype(np.float32)
+        types[::11] = -1
+        radii = rng.uniform(0.9, 2.0, n).astype(np.float32)
+        og = oracle.GridMaker(*gm_args)
+        cen = (0.3, 0, -0.1)
+        dens = og.forward(cen, coords, types, radii, T)
+        if binary:
+            dens = dens * rng.uniform(0.5, 3.0, dens.shape).astype(np.float32)
+        dens[1, 4:9] = 0
+        diff = rng.standard_normal(dens.shape).astype(np.float32)
+        ref = og.backward_relevance(cen, coords, types, radii, dens, diff)
+        scale = og.backward_relevance(cen, coords, types, radii, dens, np.abs(diff))
+        g = E.gridmaker(*gm_args)
+        rel = E.array(n, fill=5.0)
+        assert lib.mg_backward_relevance(ctypes.byref(g), 1, None, n, None, E.f3(cen),
+                                         E.ptr(E.put(coords)), E.ptr(E.put(types)), E.ptr(E.put(radii)),
+                                         T, E.ptr(E.put(dens)), E.ptr(E.put(diff)), E.ptr(rel), None) == 0
+        close_sums(rel, ref, scale, "relevance %s" % (gm_args,))
+        assert not rel[::11].any()
+    for rti in (False, True):
+        for grm in (1.0, -1.5):
+            rng = np.random.default_rng(32)
+            n, T = 40, 4
+            coords = rng.uniform(-4, 4, (n, 3)).astype(np.float32)
+            tv = rng.uniform(0, 1, (n, T)).astype(np.float32)
+            tv[rng.random((n, T)) < 0.4] = 0
+            radii = rng.uniform(1.0, 1.9, T if rti else n).astype(np.float32)
+            og = oracle.GridMaker(0.5, 9.5, False, rti, 1.0, grm)
+            diff = rng.standard_normal(og.grid_shape(T)).astype(np.float32)
+            w = rng.standard_normal((n, 3)).astype(np.float32)
+            v = rng.standard_normal((n, T)).astype(np.float32)
+            cen = (0, 0.2, 0)
+            dd, add, tdd = og.backward_gradients(cen, coords, tv, radii, diff, w, v)
+            sdd, sadd, _ = og.backward_gradients(cen, coords, tv, radii, np.abs(diff), np.abs(w), np.abs(v))
+            g = E.gridmaker(0.5, 9.5, False, rti, 1.0, grm)
+            g_dd, g_add, g_tdd = E.array(diff.shape, fill=9.0), E.array((n, 3), fill=9.0), E.array((n, T), fill=9.0)
+            assert lib.mg_backward_gradients(ctypes.byref(g), 1, None, n, None, E.f3(cen),
+                                             E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)),
+                                             T, E.ptr(E.put(diff)), E.ptr(E.put(w)), E.ptr(E.put(v)),
+                                             E.ptr(g_dd), E.ptr(g_add), E.ptr(g_tdd), None) == 0
+            assert not g_tdd.any()
+            close_sums(g_dd, dd, np.abs(sdd) + 1.0, "diffdiff rti=%s grm=%s" % (rti, grm))
+            close_sums(g_add, add, np.abs(sadd) * 4 + 1.0, "atom_diffdiff rti=%s grm=%s" % (rti, grm))
 
 
 def interpolate(in_res, in_dim_a, out_res, out_dim_a, grids, quats, shifts, centers):
