@@ -206,6 +206,48 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
             ms, nbytes, grids_per_s=round(16 / (ms * 1e-3), 1),
             workload="configs[3]: 16 x 10,000 atoms, 28x96^3 at 0.25 A")
         del out
+    # backward pass for vector types on the same atoms (atom and type gradients): the upstream
+    # gradient 16 x 28 x 96^3 is read once
+    gv = mg.GridMaker(0.25, 23.75)
+    vdiff = torch.randn((16,) + gv.grid_dimensions(28), device="cuda",
+                        generator=torch.Generator(device="cuda").manual_seed(3))
+    vag, vtg = torch.empty_like(vc), torch.empty_like(vt)
+    ms = event_ms(lambda: gv.backward_batch(ab, vcen, vc, vt, vr, vdiff, vag, vtg), 3, warmup=1)
+    res["backward_vector"] = entry(
+        ms, vdiff.numel() * 4 + vc.shape[0] * (16 + 4 * 28) + vc.shape[0] * (12 + 4 * 28),
+        atom_grads_per_s=round(vc.shape[0] / (ms * 1e-3), 1),
+        workload="configs[3] atoms: atom + type gradients against a N(0,1) gradient 16x28x96^3")
+    del vdiff, vag, vtg
+    # the autograd layer of the reference's training loop (python/torch_bindings.py:102-136) on the
+    # configuration-1 atoms as a padded batch with one-hot type vectors: forward + backward
+    from libmolgrid_amd.torch_bindings import Coords2Grid
+    off = offsets.host
+    width = int(np.diff(off).max())
+    pc = torch.zeros((B, width, 3), device="cuda")
+    pt = torch.zeros((B, width, K), device="cuda")
+    pr = torch.zeros((B, width), device="cuda")
+    ti = types.long().clamp(min=0)
+    for b in range(B):
+        n = int(off[b + 1] - off[b])
+        sl = slice(int(off[b]), int(off[b + 1]))
+        pc[b, :n], pr[b, :n] = moved[sl], radii[sl]
+        pt[b, torch.arange(n, device="cuda"), ti[sl]] = 1.0
+    layer = Coords2Grid(gm)
+    pc.requires_grad_(True)
+    upstream = src                                # any (B,K,D,D,D) tensor of values
+
+    def c2g():
+        g_out = layer(pc, pt, pr)
+        g_out.backward(upstream)
+        pc.grad = None
+
+    ms = event_ms(c2g, 5, warmup=2)
+    res["coords2grid_fwd_bwd"] = entry(
+        ms, 2 * upstream.numel() * 4 + n_atoms * (16 + 4 * K) * 2,
+        grids_per_s=round(B / (ms * 1e-3), 1),
+        workload="Coords2Grid layer, padded batch %d x %d atoms, one-hot %d-type vectors, 28x48^3: "
+                 "forward + backward (atom and type gradients)" % (B, width, K))
+    del pc, pt, pr
     # the same atoms with radii by type instead of by atom (a density per atom AND channel: no
     # matrix product, 28 times the density evaluations)
     gv = mg.GridMaker(0.25, 23.75, False, True)

@@ -575,6 +575,7 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
       const float rec_w = BINARY ? ar2 : 1.0f / ar2;
       // squared reach, with the slack that keeps the cull a superset of the exact test
       const float reach2 = (BINARY ? ar2 : frm2 * ar2) * kCullSlack;
+      const float core2 = grm2 * ar2 * kCullSlack;            // squared radius of the Gaussian core
       const float ex = fmaxf(fmaxf(clx - rec_x, rec_x - chx), 0.f);
       unsigned mask[COLS];
       unsigned any = 0;
@@ -590,6 +591,18 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
           const float bottom = (rec_z - rz - clz) * inv_block - (0.75f + 1e-3f);
           const int qhi = min((int)floorf(top), last_block), qlo = max((int)ceilf(bottom), 0);
           if (qlo <= qhi) mask[col] = (2u << qhi) - (1u << qlo);
+          if (!BINARY && !EXACT) {
+            // bits 16..27: the blocks that the Gaussian core of the atom (u <= grm^2) can reach,
+            // a subset of the above; the others take the quadratic tail without the exponential
+            const float cz2 = core2 - (ex * ex + ey * ey);
+            if (cz2 >= 0.f) {
+              const float cz = __builtin_amdgcn_sqrtf(cz2);
+              const float ctop = (rec_z + cz - clz) * inv_block + 1e-3f;
+              const float cbottom = (rec_z - cz - clz) * inv_block - (0.75f + 1e-3f);
+              const int chi = min((int)floorf(ctop), last_block), clo = max((int)ceilf(cbottom), 0);
+              if (clo <= chi) mask[col] |= (((2u << chi) - (1u << clo)) & mask[col]) << 16;
+            }
+          }
         }
         any |= mask[col];
       }
@@ -628,7 +641,8 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
         const float dx = vx - rx;
 #pragma unroll
         for (int col = 0; col < COLS; ++col) {
-          const unsigned reach = (unsigned)__builtin_amdgcn_readlane((int)mask[col], src);
+          const unsigned both = (unsigned)__builtin_amdgcn_readlane((int)mask[col], src);
+          const unsigned reach = both & 0xffffu, core = both >> 16;
           if (reach == 0) continue;
           touched |= 1u << col;
           const float dy = vy[col] - ry;
@@ -662,10 +676,14 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
               } else {
                 const float u = fmaf(dz, dz, dxy2) * rw;
                 if (u <= frm2) {
-                  const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
                   const float su = __builtin_amdgcn_sqrtf(u);
-                  const float quad = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
-                  acc[col][q] += (u <= grm2) ? gauss : quad;
+                  float val = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+                  if ((core >> q) & 1u) {          // scalar test: else no voxel of the block
+                    keep_branch();
+                    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);   // is in the core
+                    val = (u <= grm2) ? gauss : val;
+                  }
+                  acc[col][q] += val;
                 }
               }
             }

@@ -22,6 +22,11 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Inside a branch on a scalar condition: keeps the compiler from turning the branch into
+// unconditional code plus a select (it would for a few cheap-looking instructions, among them the
+// transcendental ones this is used to skip).
+__device__ __forceinline__ void keep_branch() { asm volatile(""); }
+
 // Between the LDS writes of a wave and its own reads of what other lanes wrote (and the other
 // way round).  The lanes of a wave execute an instruction together and the LDS keeps the order of
 // a wave's accesses, so the hardware needs no instruction here; this only keeps the compiler from
