@@ -517,3 +517,21 @@ def test_batch_drivers_equal_single_calls():
         assert np.array_equal(grads[s], g.backward(centers[b], coords[s], types[s], radii[s],
                                                    diff[b]))
     assert not out[1].any()
+
+
+def test_oracle_is_clean_under_address_and_ub_sanitizers():
+    """`make -C oracle asan`: every entry point of the oracle over the edge cases of its loops
+    (atoms outside the grid and on its faces, radii <= 0, ignored types, no atoms, a one-voxel
+    grid, resampling taps outside the input) in a host build with AddressSanitizer and UBSan."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ)
+    env.pop("LD_PRELOAD", None)          # the sanitizer runtime has to come first in the process
+    p = subprocess.run(["make", "-B", "-C", os.path.join(root, "oracle"), "asan"], env=env,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    if p.returncode != 0 and ("cannot find -lasan" in p.stdout or "libasan" in p.stdout
+                              and "No such file" in p.stdout):
+        pytest.skip("no sanitizer runtime for the host compiler")
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert "status 0" in p.stdout
