@@ -75,6 +75,15 @@ const char* mg_error_string(int code);
 /* Library version (major*10000 + minor*100 + patch). */
 int mg_version(void);
 
+/* No counterpart in the reference (which has no tracing, only -lineinfo,
+ * CMakeLists.txt:74).  on != 0: every entry point that launches kernels wraps
+ * its work in a roctx range named after itself (roctxRangePushA / roctxRangePop
+ * of libroctx64.so, looked up at run time), so that a rocprofv3 marker trace
+ * shows which call a kernel belongs to.  Returns the previous setting, or
+ * MG_ERR_UNSUPPORTED when the marker library cannot be loaded.  Process-wide;
+ * off by default. */
+int mg_trace_ranges(int on);
+
 /* Transform::forward on device coordinates; replaces
  * transform_forward_kernel + its launcher (src/transform.cu:13-32, 66-75).
  * out = rotate_q(in - center) + center + translation; `dotranslate` = 0 drops

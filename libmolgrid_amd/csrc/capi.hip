@@ -3,6 +3,9 @@
 // mg_forward_index keeps per device and stream (mg_forward_index_ws takes the caller's instead).
 #include <cmath>
 #include <cstdint>
+#include <dlfcn.h>
+
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -76,11 +79,45 @@ int check_common(const mg_gridmaker* g, int nbatch, const int32_t* offsets, int 
 
 int from_hip(hipError_t e) { return e == hipSuccess ? MG_OK : (int)e; }
 
+// Optional roctx ranges around the entry points (mg_trace_ranges): the marker library is looked up
+// at run time, so the library does not depend on it.
+typedef int (*RangePush)(const char*);
+typedef int (*RangePop)(void);
+std::atomic<int> g_trace{0};
+RangePush g_range_push = nullptr;
+RangePop g_range_pop = nullptr;
+
+struct Range {
+  bool on;
+  explicit Range(const char* name) : on(g_trace.load(std::memory_order_relaxed) != 0) {
+    if (on) g_range_push(name);
+  }
+  ~Range() {
+    if (on) g_range_pop();
+  }
+};
+
 }  // namespace
 
 extern "C" {
 
 int mg_version(void) { return 200; }
+
+int mg_trace_ranges(int on) {
+  static std::mutex m;
+  std::lock_guard<std::mutex> lock(m);
+  if (on && g_range_push == nullptr) {
+    void* lib = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) lib = dlopen("libroctx64.so.4", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) return MG_ERR_UNSUPPORTED;
+    RangePush push = reinterpret_cast<RangePush>(dlsym(lib, "roctxRangePushA"));
+    RangePop pop = reinterpret_cast<RangePop>(dlsym(lib, "roctxRangePop"));
+    if (push == nullptr || pop == nullptr) return MG_ERR_UNSUPPORTED;
+    g_range_pop = pop;
+    g_range_push = push;
+  }
+  return g_trace.exchange(on ? 1 : 0);
+}
 
 const char* mg_error_string(int code) {
   switch (code) {
@@ -131,6 +168,7 @@ int mg_transform_forward(int nbatch, const int32_t* atom_offsets, int atoms_per_
                          const float center_host[3], const float* translations,
                          const float translation_host[3], int dotranslate,
                          const float* in_coords, float* out_coords, void* stream) {
+  const Range range("mg_transform_forward");
   if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
     return MG_ERR_INVALID_ARGUMENT;
   if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
@@ -147,6 +185,7 @@ int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per
                           const float center_host[3], const float* translations,
                           const float translation_host[3], int dotranslate,
                           const float* in_coords, float* out_coords, void* stream) {
+  const Range range("mg_transform_backward");
   if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
     return MG_ERR_INVALID_ARGUMENT;
   if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
@@ -225,6 +264,7 @@ int mg_forward_index_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_o
                         const float grid_center_host[3], const float* coords,
                         const float* type_index, const float* radii, int ntypes, float* out,
                         void* workspace, size_t workspace_bytes, void* stream) {
+  const Range range("mg_forward_index_ws");
   bool nothing = false;
   const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
                                     radii, ntypes, out, &nothing);
@@ -243,6 +283,7 @@ int mg_forward_index_sort(const mg_gridmaker* g, int nbatch, const int32_t* atom
                           const float grid_center_host[3], const float* coords,
                           const float* type_index, const float* radii, int ntypes,
                           void* workspace, size_t workspace_bytes, void* stream) {
+  const Range range("mg_forward_index_sort");
   bool nothing = false;
   const float* const no_grid = reinterpret_cast<const float*>(16);    // only tested against NULL
   const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
@@ -264,6 +305,7 @@ int mg_forward_index_sort(const mg_gridmaker* g, int nbatch, const int32_t* atom
 int mg_forward_index_splat(const mg_gridmaker* g, int nbatch, int atoms_per_example, int ntypes,
                            float* out, const void* workspace, size_t workspace_bytes,
                            void* stream) {
+  const Range range("mg_forward_index_splat");
   int s = check_common(g, nbatch, nullptr, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
@@ -285,6 +327,7 @@ int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offs
                      const float grid_center_host[3], const float* coords,
                      const float* type_index, const float* radii, int ntypes, float* out,
                      void* stream) {
+  const Range range("mg_forward_index");
   bool nothing = false;
   const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
                                     radii, ntypes, out, &nothing);
@@ -350,6 +393,7 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
                             const float grid_center_host[3], const float* coords,
                             const float* type_index, const float* radii, int ntypes, float* out,
                             void* stream) {
+  const Range range("mg_forward_index_static");
   bool nothing = false;
   const int s = check_forward_index(g, nbatch, atom_offsets, atoms_per_example, coords, type_index,
                                     radii, ntypes, out, &nothing);
@@ -373,6 +417,7 @@ int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
                       const float grid_center_host[3], const float* coords,
                       const float* type_vector, const float* radii, int ntypes, float* out,
                       void* stream) {
+  const Range range("mg_forward_vector");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (nbatch == 0 || ntypes == 0) return MG_OK;
@@ -394,6 +439,7 @@ int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
                       const float grid_center_host[3], const float* coords,
                       const float* type_index, const float* radii, int ntypes,
                       const float* diff, float* atom_gradients, void* stream) {
+  const Range range("mg_backward_index");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   // src/grid_maker.cpp:442-444
@@ -416,6 +462,7 @@ int mg_backward_index_unrotated(const mg_gridmaker* g, int nbatch, const int32_t
                                 const float* diff, const float* quats, const float quat_host[4],
                                 const float* rot_centers, const float rot_center_host[3],
                                 float* atom_gradients, void* stream) {
+  const Range range("mg_backward_index_unrotated");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
@@ -436,6 +483,7 @@ int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
                        const float* type_vector, const float* radii, int ntypes,
                        const float* diff, float* atom_gradients, float* type_gradients,
                        void* stream) {
+  const Range range("mg_backward_vector");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
@@ -456,6 +504,7 @@ int mg_backward_relevance(const mg_gridmaker* g, int nbatch, const int32_t* atom
                           const float* type_index, const float* radii, int ntypes,
                           const float* density, const float* diff, float* relevance,
                           void* stream) {
+  const Range range("mg_backward_relevance");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
@@ -477,6 +526,7 @@ int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom
                           const float* diff, const float* atom_gradients,
                           const float* type_gradients, float* diffdiff, float* atom_diffdiff,
                           float* type_diffdiff, void* stream) {
+  const Range range("mg_backward_gradients");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   // src/grid_maker.cpp:559
@@ -498,12 +548,14 @@ int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom
 }
 
 int mg_widen(const float* src, double* dst, size_t n, void* stream) {
+  const Range range("mg_widen");
   if (n == 0) return MG_OK;
   if (src == nullptr || dst == nullptr) return MG_ERR_NULL_POINTER;
   return from_hip(launch_widen(src, dst, n, (hipStream_t)stream));
 }
 
 int mg_narrow(const double* src, float* dst, size_t n, void* stream) {
+  const Range range("mg_narrow");
   if (n == 0) return MG_OK;
   if (src == nullptr || dst == nullptr) return MG_ERR_NULL_POINTER;
   return from_hip(launch_narrow(src, dst, n, (hipStream_t)stream));
@@ -516,6 +568,7 @@ int mg_interpolate(float in_resolution, float in_dimension, float out_resolution
                    const float rot_center_host[3], const float* translations,
                    const float translation_host[3], const float* out_centers,
                    const float out_center_host[3], float* out, void* stream) {
+  const Range range("mg_interpolate");
   if (nbatch < 0 || channels < 0) return MG_ERR_INVALID_ARGUMENT;
   if (!(in_resolution > 0.f) || !(out_resolution > 0.f)) return MG_ERR_INVALID_ARGUMENT;
   // src/grid_interpolater.cpp:58-60, 70-75

@@ -174,3 +174,20 @@ def test_coordinate_set(mg):
     assert cv.has_vector_types() and cv.num_types() == 2 and len(cv) == 2
     with pytest.raises(ValueError):
         mg.CoordinateSet(c, np.zeros(3, np.float32), np.ones(2, np.float32), 2)
+
+
+def test_trace_ranges_switch():
+    """mg_trace_ranges loads the marker library at run time and wraps the entry points in roctx
+    ranges; an entry point called with ranges on behaves as before (here: an empty call)."""
+    from libmolgrid_amd import _capi
+    lib = _capi.lib
+    before = lib.mg_trace_ranges(1)
+    if before == _capi.MG_ERR_UNSUPPORTED:
+        pytest.skip("libroctx64.so is not installed")
+    try:
+        assert lib.mg_trace_ranges(1) == 1
+        assert lib.mg_transform_forward(0, None, 0, None, _capi.f4((1, 0, 0, 0)), None,
+                                        _capi.f3((0, 0, 0)), None, _capi.f3((0, 0, 0)), 1, None,
+                                        None, None) == 0
+    finally:
+        lib.mg_trace_ranges(before)
