@@ -202,6 +202,24 @@ int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
                       const float* type_vector, const float* radii, int ntypes, float* out,
                       void* stream);
 
+/* The same with an optional workspace in device memory (256-byte aligned,
+ * mg_forward_vector_workspace_size() bytes, contents undefined before and
+ * after; NULL or too small: as mg_forward_vector).  With it, a launch before
+ * the splat lists, for every example and slab of four x planes, the atoms that
+ * can reach the slab, and the workgroups of the splat scan their slab's list
+ * -- about a fifth of an example at 0.25 A -- instead of every atom of the
+ * example (the reference's kernel scans them all per block,
+ * src/grid_maker.cu:348-441).  The grids are the same bit for bit; the size is 0
+ * for the configurations that do not use lists (type-indexed radii, truncated
+ * densities).  `atoms_per_example` must be at least the largest example. */
+int mg_forward_vector_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                         int atoms_per_example, const float* grid_centers,
+                         const float grid_center_host[3], const float* coords,
+                         const float* type_vector, const float* radii, int ntypes, float* out,
+                         void* workspace, size_t workspace_bytes, void* stream);
+size_t mg_forward_vector_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
+                                        int ntypes);
+
 /* GridMaker::backward, index types; replaces set_atom_gradients and its
  * launcher (src/grid_maker.cu:472-510, 576-595), values of
  * src/grid_maker.cpp:436-467.

@@ -20,7 +20,8 @@ EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_trace_ranges", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
     "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_index_paged",
-    "mg_forward_index_sort", "mg_forward_index_splat", "mg_forward_vector", "mg_backward_index",
+    "mg_forward_index_sort", "mg_forward_index_splat", "mg_forward_vector_ws",
+    "mg_forward_vector_workspace_size", "mg_forward_vector", "mg_backward_index",
     "mg_backward_index_unrotated",
     "mg_backward_vector", "mg_backward_relevance", "mg_backward_gradients", "mg_interpolate", "mg_interpolate_force_gather",
     "mg_narrow", "mg_widen",
@@ -79,6 +80,9 @@ def declare(lib):
     lib.mg_forward_index_workspace_size.argtypes = [gm, _i, _i, _i]
     lib.mg_forward_index_workspace_size.restype = ctypes.c_size_t
     lib.mg_forward_vector.argtypes = fwd
+    lib.mg_forward_vector_ws.argtypes = fwd[:-1] + [_vp, ctypes.c_size_t, _vp]
+    lib.mg_forward_vector_workspace_size.argtypes = [gm, _i, _i, _i]
+    lib.mg_forward_vector_workspace_size.restype = ctypes.c_size_t
     lib.mg_backward_index.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp, _vp, _vp]
     lib.mg_backward_index_unrotated.argtypes = [gm, _i, _vp, _i, _vp, _f3, _vp, _vp, _vp, _i, _vp,
                                                 _vp, _f4, _vp, _f3, _vp, _vp]
@@ -97,7 +101,8 @@ def declare(lib):
     lib.mg_trace_ranges.argtypes = [_i]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)
-        if name not in ("mg_error_string", "mg_forward_index_workspace_size"):
+        if name not in ("mg_error_string", "mg_forward_index_workspace_size",
+                        "mg_forward_vector_workspace_size"):
             fn.restype = _i
     return lib
 

@@ -412,11 +412,19 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
 
 int mg_forward_index_paged(int on) { return set_forward_paged(on); }
 
-int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
-                      int atoms_per_example, const float* grid_centers,
-                      const float grid_center_host[3], const float* coords,
-                      const float* type_vector, const float* radii, int ntypes, float* out,
-                      void* stream) {
+size_t mg_forward_vector_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
+                                        int ntypes) {
+  if (g == nullptr || nbatch <= 0 || ntypes <= 0 || atoms_per_example <= 0) return 0;
+  // only the matrix-core kernel (per-atom radii, density reaching zero at the cut-off) uses lists
+  if (g->radii_type_indexed || needs_exact(g)) return 0;
+  return forward_vector_workspace_bytes(nbatch, atoms_per_example, (int)g->dim);
+}
+
+int mg_forward_vector_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                         int atoms_per_example, const float* grid_centers,
+                         const float grid_center_host[3], const float* coords,
+                         const float* type_vector, const float* radii, int ntypes, float* out,
+                         void* workspace, size_t workspace_bytes, void* stream) {
   const Range range("mg_forward_vector");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
@@ -426,12 +434,24 @@ int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
   if (has_atoms && (coords == nullptr || type_vector == nullptr || radii == nullptr))
     return MG_ERR_NULL_POINTER;
   if (g->radii_type_indexed && radii == nullptr) return MG_ERR_NULL_POINTER;
+  if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+    return MG_ERR_INVALID_ARGUMENT;
   BatchArg batch{atom_offsets, atoms_per_example};
   return from_hip(launch_forward_vector(grid_arg(g, ntypes), batch, nbatch,
                                         vec3(grid_centers, grid_center_host), coords,
                                         type_vector, radii, out, g->binary != 0,
-                                        g->radii_type_indexed != 0, needs_exact(g),
-                                        (hipStream_t)stream));
+                                        g->radii_type_indexed != 0, needs_exact(g), workspace,
+                                        workspace_bytes, (hipStream_t)stream));
+}
+
+int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
+                      int atoms_per_example, const float* grid_centers,
+                      const float grid_center_host[3], const float* coords,
+                      const float* type_vector, const float* radii, int ntypes, float* out,
+                      void* stream) {
+  return mg_forward_vector_ws(g, nbatch, atom_offsets, atoms_per_example, grid_centers,
+                              grid_center_host, coords, type_vector, radii, ntypes, out, nullptr, 0,
+                              stream);
 }
 
 int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,

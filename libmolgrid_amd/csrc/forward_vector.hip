@@ -260,12 +260,12 @@ hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nb
                                  const Vec3Arg& centers, const float* coords,
                                  const float* type_vector, const float* radii, float* out,
                                  bool binary, bool radii_type_indexed, bool exact,
-                                 hipStream_t stream) {
+                                 void* workspace, size_t workspace_bytes, hipStream_t stream) {
   // per-atom radii take the matrix-core kernel; type-indexed radii and the exact-predicate modes
   // (truncated Gaussian) use the cubic-tile kernel below
   if (!radii_type_indexed && !exact)
     return launch_forward_vector_mfma(g, batch, nbatch, centers, coords, type_vector, radii, out,
-                                      binary, stream);
+                                      binary, workspace, workspace_bytes, stream);
   if (binary && radii_type_indexed)
     return launch_sized<true, true>(g, batch, nbatch, centers, coords, type_vector, radii, out, exact, stream);
   if (binary)

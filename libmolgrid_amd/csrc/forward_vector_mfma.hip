@@ -70,7 +70,8 @@ __global__ __launch_bounds__(kColThreads) __attribute__((amdgpu_waves_per_eu(3, 
 splat_vector_mfma_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_vector, const float* __restrict__ radii,
-    float* __restrict__ out, int cols_per_side, int vec_store, int vec_weights) {
+    float* __restrict__ out, int cols_per_side, int vec_store, int vec_weights,
+    const unsigned* __restrict__ slab_lists, const int* __restrict__ slab_counts, int list_stride) {
   __shared__ unsigned short s_idx[kColWaves][kSeg];
   __shared__ int s_wcount[kColWaves];
   // The rows of the current chunk of records while sums are formed, the stage of the write-out
@@ -135,16 +136,30 @@ splat_vector_mfma_kernel(
   int ncand = 0;
 
   // ---- scan: atoms [s0, s1) against the group's box -> per-wave index segments --------------
+  // With lists (a launch before this one has left, for every example and slab of four x planes,
+  // the atoms that can reach the slab's planes, in atom order), a workgroup scans its slab's list
+  // -- about a fifth of the example -- instead of all atoms.
+  const unsigned* const my_list =
+      slab_lists != nullptr ? slab_lists + ((size_t)b * cols_per_side + x0 / kColXY) * list_stride : nullptr;
+  const int my_listed = slab_lists != nullptr ? slab_counts[b * cols_per_side + x0 / kColXY] : 0;
   auto scan = [&](int s0, int s1) -> bool {
-    const int quarter = (s1 - s0 + kColWaves - 1) / kColWaves;
+    // what is scanned: positions [0, total) of the list, or the atoms s0 + [0, total)
+    const int total = my_list != nullptr ? my_listed : s1 - s0;
+    const int quarter = (total + kColWaves - 1) / kColWaves;
     int wcnt = 0;
-    const int wb = s0 + wave * quarter, we = min(s1, wb + quarter);
+    const int wb = wave * quarter, we = min(total, wb + quarter);
     constexpr int U = 2;
-    for (int a0 = wb; a0 < we; a0 += kWave * U) {
+    for (int i0 = wb; i0 < we; i0 += kWave * U) {
       float rr[U], cx[U], cy[U], cz[U];
+      int at[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int a = min(a0 + u * kWave + lane, we - 1);
+        const int i = min(i0 + u * kWave + lane, we - 1);
+        at[u] = my_list != nullptr ? begin + (int)my_list[i] : s0 + i;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int a = at[u];
         rr[u] = radii[a];
         cx[u] = coords[3 * a];
         cy[u] = coords[3 * a + 1];
@@ -152,10 +167,11 @@ splat_vector_mfma_kernel(
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int a = a0 + u * kWave + lane;
+        const int a = at[u];
         const float reach = rr[u] * g.radius_scale * (BINARY ? 1.0f : g.frm);
-        const bool p = (a < we) && box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy,
-                                                 chz) <= reach * reach * kCullSlack;
+        const bool p = (i0 + u * kWave + lane < we) && a >= s0 && a < s1 &&
+                       box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy, chz) <=
+                           reach * reach * kCullSlack;
         const unsigned long long m = __ballot(p);
         const int pos = wcnt + __popcll(m & ((1ull << lane) - 1ull));
         if (p && pos < kSeg) s_idx[wave][pos] = (unsigned short)(a - s0);
@@ -447,13 +463,86 @@ splat_vector_mfma_kernel(
   }
 }
 
+// The launch before the splat: for every example and slab of four x planes, the atoms whose reach
+// (their final radius; binary: their radius) comes to the slab's planes, as indices relative to the
+// example's first atom, in ascending order.  The test is the x term of the splat kernel's own box
+// test with the same floats, so the list holds every atom that kernel would have found.
+constexpr int kListThreads = 512;
+constexpr int kListWaves = kListThreads / kWave;
+template <bool BINARY>
+__global__ __launch_bounds__(kListThreads) void slab_list_kernel(
+    GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
+    const float* __restrict__ radii, unsigned* __restrict__ slab_lists,
+    int* __restrict__ slab_counts, int list_stride) {
+  __shared__ int s_wave_count[kListWaves];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int xs = blockIdx.x, b = blockIdx.y, nxs = gridDim.x;
+  int begin, end;
+  example_range(batch, b, begin, end);
+  const float ox = load3(centers, b).x - g.half_dimension;
+  const float clx = grid_coord(ox, xs * kColXY, g.resolution);
+  const float chx = grid_coord(ox, min(xs * kColXY + kColXY, g.dim) - 1, g.resolution);
+  unsigned* const list = slab_lists + ((size_t)b * nxs + xs) * list_stride;
+  int listed = 0;
+  for (int a0 = begin; a0 < end; a0 += kListThreads) {
+    const int a = a0 + tid;
+    bool p = false;
+    if (a < end) {
+      const float x = coords[3 * a];
+      const float reach = radii[a] * g.radius_scale * (BINARY ? 1.0f : g.frm);
+      const float ex = fmaxf(fmaxf(clx - x, x - chx), 0.f);
+      p = sq_distance_exact(ex, 0.f, 0.f) <= reach * reach * kCullSlack;
+    }
+    const unsigned long long m = __ballot(p);
+    if (lane == 0) s_wave_count[wave] = __popcll(m);
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kListWaves; ++w) {
+      const int c = s_wave_count[w];
+      before += w < wave ? c : 0;
+      all += c;
+    }
+    const int pos = listed + before + __popcll(m & ((1ull << lane) - 1ull));
+    if (p && pos < list_stride) list[pos] = (unsigned)(a - begin);
+    listed += all;
+    __syncthreads();
+  }
+  if (tid == 0) slab_counts[b * nxs + xs] = min(listed, list_stride);
+}
+
 }  // namespace
+
+size_t forward_vector_workspace_bytes(int nbatch, int atoms_per_example, int dim) {
+  const size_t nxs = (size_t)((dim + kColXY - 1) / kColXY);
+  return ((nbatch * nxs * sizeof(int) + 255) & ~(size_t)255) +
+         (size_t)nbatch * nxs * (size_t)atoms_per_example * sizeof(unsigned);
+}
 
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
                                       const Vec3Arg& centers, const float* coords,
                                       const float* type_vector, const float* radii, float* out,
-                                      bool binary, hipStream_t stream) {
+                                      bool binary, void* workspace, size_t workspace_bytes,
+                                      hipStream_t stream) {
   const int cols_per_side = (g.dim + kColXY - 1) / kColXY;
+  // per-slab atom lists, when the caller has brought the memory for them and the example has atoms
+  unsigned* lists = nullptr;
+  int* counts = nullptr;
+  const int list_stride = batch.per_example;
+  if (workspace != nullptr && list_stride > 0 &&
+      workspace_bytes >= forward_vector_workspace_bytes(nbatch, list_stride, g.dim)) {
+    counts = static_cast<int*>(workspace);
+    lists = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(workspace) +
+                                        (((size_t)nbatch * cols_per_side * sizeof(int) + 255) & ~(size_t)255));
+    if (binary)
+      hipLaunchKernelGGL(slab_list_kernel<true>, dim3(cols_per_side, nbatch), dim3(kListThreads), 0,
+                         stream, g, batch, centers, coords, radii, lists, counts, list_stride);
+    else
+      hipLaunchKernelGGL(slab_list_kernel<false>, dim3(cols_per_side, nbatch), dim3(kListThreads), 0,
+                         stream, g, batch, centers, coords, radii, lists, counts, list_stride);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
   const int slabs = (g.dim + kSlabZ - 1) / kSlabZ;
   const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
   const int vec_store = ((g.dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0) &&
@@ -464,11 +553,11 @@ hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, i
   if (binary)
     hipLaunchKernelGGL(splat_vector_mfma_kernel<true>, dim3(groups * slabs, nbatch),
                        dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
-                       out, cols_per_side, vec_store, vec_weights);
+                       out, cols_per_side, vec_store, vec_weights, lists, counts, list_stride);
   else
     hipLaunchKernelGGL(splat_vector_mfma_kernel<false>, dim3(groups * slabs, nbatch),
                        dim3(kColThreads), 0, stream, g, batch, centers, coords, type_vector, radii,
-                       out, cols_per_side, vec_store, vec_weights);
+                       out, cols_per_side, vec_store, vec_weights, lists, counts, list_stride);
   return hipGetLastError();
 }
 

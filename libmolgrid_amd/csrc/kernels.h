@@ -55,16 +55,21 @@ hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_examp
 int set_forward_paged(int on);
 
 // vector types with per-atom radii, density mode, on the matrix cores (forward_vector_mfma.hip)
+// `workspace` (optional, forward_vector_workspace_bytes()): a launch before the splat leaves the
+// atoms that can reach each slab of four x planes there, and the splat's workgroups scan their
+// slab's list instead of every atom of their example.  Same grids either way.
+size_t forward_vector_workspace_bytes(int nbatch, int atoms_per_example, int dim);
 hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, int nbatch,
                                       const Vec3Arg& centers, const float* coords,
                                       const float* type_vector, const float* radii, float* out,
-                                      bool binary, hipStream_t stream);
+                                      bool binary, void* workspace, size_t workspace_bytes,
+                                      hipStream_t stream);
 
 hipError_t launch_forward_vector(const GridArg& g, const BatchArg& batch, int nbatch,
                                  const Vec3Arg& centers, const float* coords,
                                  const float* type_vector, const float* radii, float* out,
                                  bool binary, bool radii_type_indexed, bool exact,
-                                 hipStream_t stream);
+                                 void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nbatch,
                                  int launch_atoms, const Vec3Arg& centers, const float* coords,

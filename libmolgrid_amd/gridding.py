@@ -1134,22 +1134,28 @@ class GridMaker(object):
                 raise IndexError("Type index %d larger than allowed %d"
                                  % (int(np.floor(t).max()), ntypes))
 
-    def _forward_index_call(self, batch=None):
-        """mg_forward_index_ws with a workspace from torch's allocator (which is stream aware); a
-        ragged batch layout (AtomBatch) keeps its workspace for the next call."""
+    def _forward_index_call(self, batch=None, vector=False):
+        """mg_forward_index_ws (mg_forward_vector_ws) with a workspace from torch's allocator
+        (which is stream aware); a ragged batch layout (AtomBatch) keeps its workspace for the
+        next call."""
+        size_of = _lib.mg_forward_vector_workspace_size if vector else \
+            _lib.mg_forward_index_workspace_size
+        entry = _lib.mg_forward_vector_ws if vector else _lib.mg_forward_index_ws
+        name = "forward_vector_ws" if vector else "forward_index_ws"
+
         def call(p, B, off, n, cen, chost, coords, types, radii, T, out, stream):
-            need = int(_lib.mg_forward_index_workspace_size(p, B, n, T))
+            need = int(size_of(p, B, n, T))
             ws = None
             if need:
                 # one workspace per device AND stream: calls on two streams may overlap
-                key = ("forward_index_ws", torch.cuda.current_device(), stream)
+                key = (name, torch.cuda.current_device(), stream)
                 ws = batch.scratch.get(key) if batch is not None else None
                 if ws is None or ws.numel() < need:
                     ws = torch.empty(need, dtype=torch.uint8, device=_device())
                     if batch is not None:
                         batch.scratch[key] = ws
-            return _lib.mg_forward_index_ws(p, B, off, n, cen, chost, coords, types, radii, T, out,
-                                            ws.data_ptr() if ws is not None else None, need, stream)
+            return entry(p, B, off, n, cen, chost, coords, types, radii, T, out,
+                         ws.data_ptr() if ws is not None else None, need, stream)
         return call
 
     # -- forward ------------------------------------------------------------
@@ -1209,7 +1215,7 @@ class GridMaker(object):
             fn = self._forward_index_call()
         else:
             self._check_vector_args(n, a_types, a_radii, a_out.shape)
-            fn = _lib.mg_forward_vector
+            fn = self._forward_index_call(vector=True)
         code = fn(self._p, 1, None, n, None, _capi.f3(c), a_coords.ptr, a_types.ptr, a_radii.ptr,
                   a_out.shape[0], a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward")
@@ -1301,7 +1307,7 @@ class GridMaker(object):
         else:
             self._check_vector_args(n, _Shape(a_types.shape[1:]), _Shape(a_radii.shape[1:]),
                                     a_out.shape[1:])
-            fn = _lib.mg_forward_vector
+            fn = self._forward_index_call(vector=True)
         code = fn(self._p, B, None, n, None if one_center else a_centers.ptr, chost, a_coords.ptr,
                   a_types.ptr, a_radii.ptr, a_out.shape[1], a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward")
@@ -1341,7 +1347,8 @@ class GridMaker(object):
                 raise IndexError("radii does not match number of types")
             if not rti and a_radii.shape[0] < total:
                 raise IndexError("radii does not match number of atoms")
-            fn = _lib.mg_forward_vector
+            fn = self._forward_index_call(offsets if isinstance(offsets, AtomBatch) else None,
+                                          vector=True)
         code = fn(self._p, B, _ptr(off), largest, _ptr(cen), _capi.f3(_Z3), a_coords.ptr,
                   a_types.ptr, a_radii.ptr, T, a_out.ptr, _stream())
         _capi.check(code, "GridMaker.forward_batch")

@@ -318,13 +318,19 @@ def vector_case(rng, natoms, ntypes, extent, sparse=0.5):
     return coords, tv, radii
 
 
-def forward_vector(gm_args, center, coords, tv, radii):
+def forward_vector(gm_args, center, coords, tv, radii, lists=False):
+    """lists: with the workspace for per-slab atom lists (mg_forward_vector_ws)"""
     g = E.gridmaker(*gm_args)
     dim, ntypes = int(g.dim), tv.shape[1]
     out = E.array((ntypes, dim, dim, dim), fill=3.0)
-    code = lib.mg_forward_vector(ctypes.byref(g), 1, None, len(coords), None, E.f3(center),
-                                 E.ptr(E.put(coords)), E.ptr(E.put(tv)), E.ptr(E.put(radii)), ntypes,
-                                 E.ptr(out), None)
+    args = [ctypes.byref(g), 1, None, len(coords), None, E.f3(center), E.ptr(E.put(coords)),
+            E.ptr(E.put(tv)), E.ptr(E.put(radii)), ntypes, E.ptr(out)]
+    if lists:
+        need = lib.mg_forward_vector_workspace_size(ctypes.byref(g), 1, len(coords), ntypes)
+        ws = E.array(need, np.uint8, tight=False) if need else None
+        code = lib.mg_forward_vector_ws(*args, E.ptr(ws), need, None)
+    else:
+        code = lib.mg_forward_vector(*args, None)
     assert code == 0, code
     return out
 
@@ -353,6 +359,34 @@ def group_forward_vector():
         ref = oracle.GridMaker(0.5, 9.5, binary, True).forward((0, 0, 0), coords, tv, tr)
         got = forward_vector((0.5, 9.5, binary, True), (0, 0, 0), coords, tv, tr)
         close(got, ref, "vector forward, radii by type, binary=%s" % binary, exact=binary)
+    # per-slab atom lists: the same grids bit for bit, also for a batch with an empty example and
+    # for more atoms than one scan pass holds per wave (several passes over the list)
+    for ntypes, natoms, dimension in ((5, 60, 11.5), (28, 300, 15.5), (3, 6000, 9.5)):
+        for binary in (False, True):
+            rng = np.random.default_rng(200 + natoms)
+            coords, tv, radii = vector_case(rng, natoms, ntypes, dimension / 2 + 1.0)
+            plain = forward_vector((0.5, dimension, binary), (0.1, 0, 0), coords, tv, radii).copy()
+            listed = forward_vector((0.5, dimension, binary), (0.1, 0, 0), coords, tv, radii, lists=True)
+            close(listed, plain, "atom lists T=%d n=%d binary=%s" % (ntypes, natoms, binary), exact=True)
+    rng = np.random.default_rng(14)
+    coords, tv, radii = vector_case(rng, 130, 4, 6.5)
+    off = np.array([0, 50, 50, 130], np.int32)
+    g = E.gridmaker(0.5, 11.5)
+    dim = int(g.dim)
+    cen = E.put(rng.uniform(-1, 1, (3, 3)).astype(np.float32))
+    outs = []
+    for use in (False, True):
+        need = lib.mg_forward_vector_workspace_size(ctypes.byref(g), 3, 80, 4) if use else 0
+        ws = E.array(need, np.uint8, tight=False) if need else None
+        out = E.array((3, 4, dim, dim, dim), fill=3.0)
+        assert lib.mg_forward_vector_ws(ctypes.byref(g), 3, E.ptr(E.put(off, np.int32)), 80, E.ptr(cen),
+                                        E.f3((0, 0, 0)), E.ptr(E.put(coords)), E.ptr(E.put(tv)),
+                                        E.ptr(E.put(radii)), 4, E.ptr(out), E.ptr(ws), need, None) == 0
+        outs.append(np.array(out))
+    close(outs[1], outs[0], "atom lists, ragged batch", exact=True)
+    ref = oracle.GridMaker(0.5, 11.5).forward_batch(off.astype(np.int64), np.array(cen), coords, tv, radii, 4)
+    close(outs[1], ref, "atom lists, ragged batch vs oracle")
+    assert not outs[1][1].any()
     # a larger grid (two z slabs in the matrix-core kernel's terms): dim 60
     rng = np.random.default_rng(13)
     coords, tv, radii = vector_case(rng, 150, 4, 16.0)
