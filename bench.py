@@ -206,48 +206,54 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
             ms, nbytes, grids_per_s=round(16 / (ms * 1e-3), 1),
             workload="configs[3]: 16 x 10,000 atoms, 28x96^3 at 0.25 A")
         del out
-    # backward pass for vector types on the same atoms (atom and type gradients): the upstream
-    # gradient 16 x 28 x 96^3 is read once
-    gv = mg.GridMaker(0.25, 23.75)
-    vdiff = torch.randn((16,) + gv.grid_dimensions(28), device="cuda",
-                        generator=torch.Generator(device="cuda").manual_seed(3))
-    vag, vtg = torch.empty_like(vc), torch.empty_like(vt)
-    ms = event_ms(lambda: gv.backward_batch(ab, vcen, vc, vt, vr, vdiff, vag, vtg), 3, warmup=1)
-    res["backward_vector"] = entry(
-        ms, vdiff.numel() * 4 + vc.shape[0] * (16 + 4 * 28) + vc.shape[0] * (12 + 4 * 28),
-        atom_grads_per_s=round(vc.shape[0] / (ms * 1e-3), 1),
-        workload="configs[3] atoms: atom + type gradients against a N(0,1) gradient 16x28x96^3")
-    del vdiff, vag, vtg
-    # the autograd layer of the reference's training loop (python/torch_bindings.py:102-136) on the
-    # configuration-1 atoms as a padded batch with one-hot type vectors: forward + backward
-    from libmolgrid_amd.torch_bindings import Coords2Grid
-    off = offsets.host
-    width = int(np.diff(off).max())
-    pc = torch.zeros((B, width, 3), device="cuda")
-    pt = torch.zeros((B, width, K), device="cuda")
-    pr = torch.zeros((B, width), device="cuda")
-    ti = types.long().clamp(min=0)
-    for b in range(B):
-        n = int(off[b + 1] - off[b])
-        sl = slice(int(off[b]), int(off[b + 1]))
-        pc[b, :n], pr[b, :n] = moved[sl], radii[sl]
-        pt[b, torch.arange(n, device="cuda"), ti[sl]] = 1.0
-    layer = Coords2Grid(gm)
-    pc.requires_grad_(True)
-    upstream = src                                # any (B,K,D,D,D) tensor of values
+    try:
+        # backward pass for vector types on the same atoms (atom and type gradients): the upstream
+        # gradient 16 x 28 x 96^3 is read once
+        gv = mg.GridMaker(0.25, 23.75)
+        vdiff = torch.randn((16,) + gv.grid_dimensions(28), device="cuda",
+                            generator=torch.Generator(device="cuda").manual_seed(3))
+        vag, vtg = torch.empty_like(vc), torch.empty_like(vt)
+        ms = event_ms(lambda: gv.backward_batch(ab, vcen, vc, vt, vr, vdiff, vag, vtg), 3, warmup=1)
+        res["backward_vector"] = entry(
+            ms, vdiff.numel() * 4 + vc.shape[0] * (16 + 4 * 28) + vc.shape[0] * (12 + 4 * 28),
+            atom_grads_per_s=round(vc.shape[0] / (ms * 1e-3), 1),
+            workload="configs[3] atoms: atom + type gradients against a N(0,1) gradient 16x28x96^3")
+        del vdiff, vag, vtg
+    except Exception as e:          # a new measurement must not cost the bench line
+        res["backward_vector"] = {"error": repr(e)[:200]}
+    try:
+        # the autograd layer of the reference's training loop (python/torch_bindings.py:102-136) on the
+        # configuration-1 atoms as a padded batch with one-hot type vectors: forward + backward
+        from libmolgrid_amd.torch_bindings import Coords2Grid
+        off = offsets.host
+        width = int(np.diff(off).max())
+        pc = torch.zeros((B, width, 3), device="cuda")
+        pt = torch.zeros((B, width, K), device="cuda")
+        pr = torch.zeros((B, width), device="cuda")
+        ti = types.long().clamp(min=0)
+        for b in range(B):
+            n = int(off[b + 1] - off[b])
+            sl = slice(int(off[b]), int(off[b + 1]))
+            pc[b, :n], pr[b, :n] = moved[sl], radii[sl]
+            pt[b, torch.arange(n, device="cuda"), ti[sl]] = 1.0
+        layer = Coords2Grid(gm)
+        pc.requires_grad_(True)
+        upstream = src                                # any (B,K,D,D,D) tensor of values
 
-    def c2g():
-        g_out = layer(pc, pt, pr)
-        g_out.backward(upstream)
-        pc.grad = None
+        def c2g():
+            g_out = layer(pc, pt, pr)
+            g_out.backward(upstream)
+            pc.grad = None
 
-    ms = event_ms(c2g, 5, warmup=2)
-    res["coords2grid_fwd_bwd"] = entry(
-        ms, 2 * upstream.numel() * 4 + n_atoms * (16 + 4 * K) * 2,
-        grids_per_s=round(B / (ms * 1e-3), 1),
-        workload="Coords2Grid layer, padded batch %d x %d atoms, one-hot %d-type vectors, 28x48^3: "
-                 "forward + backward (atom and type gradients)" % (B, width, K))
-    del pc, pt, pr
+        ms = event_ms(c2g, 5, warmup=2)
+        res["coords2grid_fwd_bwd"] = entry(
+            ms, 2 * upstream.numel() * 4 + n_atoms * (16 + 4 * K) * 2,
+            grids_per_s=round(B / (ms * 1e-3), 1),
+            workload="Coords2Grid layer, padded batch %d x %d atoms, one-hot %d-type vectors, 28x48^3: "
+                     "forward + backward (atom and type gradients)" % (B, width, K))
+        del pc, pt, pr
+    except Exception as e:          # a new measurement must not cost the bench line
+        res["coords2grid_fwd_bwd"] = {"error": repr(e)[:200]}
     # the same atoms with radii by type instead of by atom (a density per atom AND channel: no
     # matrix product, 28 times the density evaluations)
     gv = mg.GridMaker(0.25, 23.75, False, True)
@@ -367,12 +373,24 @@ def main():
     write_out = {}
     if not args.no_autotune:
         from libmolgrid_amd import _capi
-        for name, on in (("per_wave", 0), ("paged", 1)):
-            _capi.lib.mg_forward_index_paged(on)
-            write_out[name + "_ms"] = round(event_ms(k_forward, max(args.steps, 10)), 4)
-        use_paged = write_out["paged_ms"] < write_out["per_wave_ms"]
+        try:
+            k_transform()
+            k_forward()
+            torch.cuda.synchronize()
+            per_wave_grid = grid.clone()
+            for name, on in (("per_wave", 0), ("paged", 1)):
+                _capi.lib.mg_forward_index_paged(on)
+                write_out[name + "_ms"] = round(event_ms(k_forward, max(args.steps, 10)), 4)
+            torch.cuda.synchronize()
+            if not torch.equal(grid, per_wave_grid):       # the paged grids: bit for bit
+                raise RuntimeError("the paged write-out gives different grids")
+            del per_wave_grid
+            use_paged = write_out["paged_ms"] < write_out["per_wave_ms"]
+            write_out["used"] = "paged" if use_paged else "per_wave"
+        except Exception as e:                             # reported; the default stays
+            use_paged = False
+            write_out["error"] = repr(e)[:200]
         _capi.lib.mg_forward_index_paged(1 if use_paged else 0)
-        write_out["used"] = "paged" if use_paged else "per_wave"
 
     step_serial()
     torch.cuda.synchronize()
@@ -401,31 +419,42 @@ def main():
     # backward pass, and launch by launch or as one captured HIP graph (nothing in a step
     # allocates or synchronises).  Every variant is checked against the serial eager step bit
     # for bit and timed over exactly --steps steps; `value` is the fastest one's, all are listed.
-    variants = {}
-    order = [("serial", step_serial)]
-    if not args.serial_only:
-        order.append(("overlapped", step_overlapped))
-    for name, fn in order:
-        grid.zero_()
-        grads.zero_()
+    variants = {"serial_eager": timed(step_serial)}
+
+    def graph_of(fn, what):
         fn()
-        same_as_serial(name + " step")
-        variants[name + "_eager"] = timed(fn)
-        if args.no_graph:
-            continue
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(2):                        # replays must reproduce the eager results
+            grid.zero_()
+            grads.zero_()
+            graph.replay()
+            same_as_serial("replay of the captured %s step" % what)
+        return graph
+
+    # (a variant that fails -- a capture the runtime refuses, a mismatch -- is reported under
+    # its name and leaves the others standing)
+    if not args.no_graph:
         try:
-            fn()                                  # workspaces exist before the capture
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                fn()
-            for _ in range(2):                    # replays must reproduce the eager results
-                graph.replay()
-                same_as_serial("replay of the captured %s step" % name)
-            variants[name + "_graph"] = timed(graph.replay)
-        except RuntimeError as e:                 # a capture that fails is reported, not fatal
-            variants[name + "_graph"] = (float("inf"), float("inf"))
-            variants[name + "_graph_error"] = str(e)[:200]
+            variants["serial_graph"] = timed(graph_of(step_serial, "serial").replay)
+        except Exception as e:
+            variants["serial_graph_error"] = repr(e)[:200]
+    if not args.serial_only:
+        try:
+            grid.zero_()
+            grads.zero_()
+            step_overlapped()
+            same_as_serial("overlapped step")
+            variants["overlapped_eager"] = timed(step_overlapped)
+            if not args.no_graph:
+                try:
+                    variants["overlapped_graph"] = timed(graph_of(step_overlapped, "overlapped").replay)
+                except Exception as e:
+                    variants["overlapped_graph_error"] = repr(e)[:200]
+        except Exception as e:
+            variants["overlapped_eager_error"] = repr(e)[:200]
     del expect
     timings = {k: v for k, v in variants.items() if isinstance(v, tuple)}
     best = min(timings, key=lambda k: timings[k][0])
