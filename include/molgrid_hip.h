@@ -15,7 +15,9 @@
  *     except mg_forward_index (see there).
  *   - Batches: example b owns atoms [atom_offsets[b], atom_offsets[b+1]) of the
  *     packed atom arrays, and `atoms_per_example` must then be at least the size
- *     of the largest example (it sizes launches and workspaces).  When
+ *     of the largest example (it sizes launches and workspaces); 0 means "no
+ *     atoms at all" for every entry point (offsets and atom arrays are then not
+ *     looked at and may be NULL), a negative value is rejected.  When
  *     `atom_offsets` is NULL every example owns `atoms_per_example` consecutive
  *     atoms (the reference's padded BxN layout,
  *     include/libmolgrid/grid_maker.h:265-301; nbatch = 1 is the un-batched

@@ -71,7 +71,7 @@ int check_common(const mg_gridmaker* g, int nbatch, const int32_t* offsets, int 
                  int ntypes) {
   if (g == nullptr) return MG_ERR_NULL_POINTER;
   if (nbatch < 0 || ntypes < 0) return MG_ERR_INVALID_ARGUMENT;
-  if (offsets == nullptr && per_example < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (per_example < 0) return MG_ERR_INVALID_ARGUMENT;
   if (g->dim == 0 || g->dim > 65535u) return MG_ERR_OUT_OF_RANGE;
   if (!(g->resolution > 0.f)) return MG_ERR_INVALID_ARGUMENT;
   return MG_OK;
@@ -169,11 +169,10 @@ int mg_transform_forward(int nbatch, const int32_t* atom_offsets, int atoms_per_
                          const float translation_host[3], int dotranslate,
                          const float* in_coords, float* out_coords, void* stream) {
   const Range range("mg_transform_forward");
-  if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
-    return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch < 0 || atoms_per_example < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (in_coords == nullptr || out_coords == nullptr) return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_transform(batch, nbatch, atoms_per_example, vec4(quats, quat_host),
                                    vec3(centers, center_host),
                                    vec3(translations, translation_host), dotranslate != 0, false,
@@ -186,11 +185,10 @@ int mg_transform_backward(int nbatch, const int32_t* atom_offsets, int atoms_per
                           const float translation_host[3], int dotranslate,
                           const float* in_coords, float* out_coords, void* stream) {
   const Range range("mg_transform_backward");
-  if (nbatch < 0 || (atom_offsets == nullptr && atoms_per_example < 0))
-    return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch < 0 || atoms_per_example < 0) return MG_ERR_INVALID_ARGUMENT;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (in_coords == nullptr || out_coords == nullptr) return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_transform(batch, nbatch, atoms_per_example, vec4(quats, quat_host),
                                    vec3(centers, center_host),
                                    vec3(translations, translation_host), dotranslate != 0, true,
@@ -430,13 +428,13 @@ int mg_forward_vector_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_
   if (s != MG_OK) return s;
   if (nbatch == 0 || ntypes == 0) return MG_OK;
   if (out == nullptr) return MG_ERR_NULL_POINTER;
-  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
+  const bool has_atoms = atoms_per_example > 0;
   if (has_atoms && (coords == nullptr || type_vector == nullptr || radii == nullptr))
     return MG_ERR_NULL_POINTER;
   if (g->radii_type_indexed && radii == nullptr) return MG_ERR_NULL_POINTER;
   if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
     return MG_ERR_INVALID_ARGUMENT;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_forward_vector(grid_arg(g, ntypes), batch, nbatch,
                                         vec3(grid_centers, grid_center_host), coords,
                                         type_vector, radii, out, g->binary != 0,
@@ -464,11 +462,11 @@ int mg_backward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
   if (s != MG_OK) return s;
   // src/grid_maker.cpp:442-444
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (coords == nullptr || type_index == nullptr || radii == nullptr || diff == nullptr ||
       atom_gradients == nullptr)
     return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_backward_index(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
                                         vec3(grid_centers, grid_center_host), coords,
                                         type_index, radii, diff, atom_gradients,
@@ -486,11 +484,11 @@ int mg_backward_index_unrotated(const mg_gridmaker* g, int nbatch, const int32_t
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (coords == nullptr || type_index == nullptr || radii == nullptr || diff == nullptr ||
       atom_gradients == nullptr)
     return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_backward_index_unrotated(
       grid_arg(g, ntypes), batch, nbatch, atoms_per_example, vec3(grid_centers, grid_center_host),
       coords, type_index, radii, diff, vec4(quats, quat_host), vec3(rot_centers, rot_center_host),
@@ -506,11 +504,11 @@ int mg_backward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_of
   const Range range("mg_backward_vector");
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (coords == nullptr || type_vector == nullptr || radii == nullptr || diff == nullptr ||
       atom_gradients == nullptr || type_gradients == nullptr)
     return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_backward_vector(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
                                          vec3(grid_centers, grid_center_host), coords,
                                          type_vector, radii, diff, atom_gradients,
@@ -528,11 +526,11 @@ int mg_backward_relevance(const mg_gridmaker* g, int nbatch, const int32_t* atom
   int s = check_common(g, nbatch, atom_offsets, atoms_per_example, ntypes);
   if (s != MG_OK) return s;
   if (g->radii_type_indexed) return MG_ERR_INVALID_ARGUMENT;
-  if (nbatch == 0 || (atom_offsets == nullptr && atoms_per_example == 0)) return MG_OK;
+  if (nbatch == 0 || atoms_per_example == 0) return MG_OK;   // no atoms at all
   if (coords == nullptr || type_index == nullptr || radii == nullptr || density == nullptr ||
       diff == nullptr || relevance == nullptr)
     return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_backward_relevance(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
                                             vec3(grid_centers, grid_center_host), coords,
                                             type_index, radii, density, diff, relevance,
@@ -553,12 +551,12 @@ int mg_backward_gradients(const mg_gridmaker* g, int nbatch, const int32_t* atom
   if (g->binary) return MG_ERR_INVALID_ARGUMENT;
   if (nbatch == 0 || ntypes == 0) return MG_OK;
   if (diffdiff == nullptr) return MG_ERR_NULL_POINTER;
-  const bool has_atoms = atom_offsets != nullptr || atoms_per_example > 0;
+  const bool has_atoms = atoms_per_example > 0;
   if (has_atoms && (coords == nullptr || type_vector == nullptr || radii == nullptr ||
                     diff == nullptr || atom_gradients == nullptr || type_gradients == nullptr ||
                     atom_diffdiff == nullptr || type_diffdiff == nullptr))
     return MG_ERR_NULL_POINTER;
-  BatchArg batch{atom_offsets, atoms_per_example};
+  BatchArg batch{atoms_per_example > 0 ? atom_offsets : nullptr, atoms_per_example};
   return from_hip(launch_backward_gradients(grid_arg(g, ntypes), batch, nbatch, atoms_per_example,
                                             vec3(grid_centers, grid_center_host), coords,
                                             type_vector, radii, diff, atom_gradients,

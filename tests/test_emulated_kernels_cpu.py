@@ -31,3 +31,14 @@ def test_group(emulated_library, group):
                        stderr=subprocess.STDOUT, text=True, timeout=1200)
     assert p.returncode == 0, "emulated %s failed (status %d):\n%s" % (group, p.returncode, p.stdout[-4000:])
     assert "comparisons passed" in p.stdout
+
+
+def test_hostile_inputs_return(emulated_library):
+    """tests/emu/fuzz.py: not-a-number and infinite coordinates, radii, types, centres and
+    quaternions, radii <= 0 and far larger than the grid, types at and beyond the channel count,
+    grids of 1 to 65 voxels a side, empty examples, 70 examples -- every kernel must return without
+    leaving its arrays and without a deadlock (a few rounds here; more by hand)."""
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "fuzz.py"), "12", "3"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+    assert p.returncode == 0, "fuzz failed (status %d):\n%s" % (p.returncode, p.stdout[-3000:])
+    assert "12 rounds returned" in p.stdout
