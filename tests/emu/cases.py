@@ -522,6 +522,41 @@ def group_interpolate():
         close(gathered, got, "gather path equals staged path", exact=True)
 
 
+def group_config0():
+    """BASELINE configuration 0 at full size (1,540 atoms into 28 x 48^3) plus one example of
+    configuration 1 (rotated, translated): forward in both write-outs, backward."""
+    lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    c0 = synth.config0()
+    c1 = synth.config1(nbatch=2)
+    moved = oracle.transform_forward_batch(c1["offsets"], c1["quats"], c1["centers"],
+                                           c1["translations"], c1["coords"])
+    s1 = slice(int(c1["offsets"][1]), int(c1["offsets"][2]))
+    for name, center, coords, types, radii in (
+            ("configuration 0", c0["centers"][0], c0["coords"], c0["types"], c0["radii"]),
+            ("configuration 1, example 1", c1["centers"][1], moved[s1], c1["types"][s1], c1["radii"][s1])):
+        og = oracle.GridMaker(0.5, 23.5)
+        ref = og.forward(center, coords, types, radii, 28)
+        plain = forward_index((0.5, 23.5), center, coords, types, radii, 28).copy()
+        lib.mg_forward_index_paged(1)
+        paged = forward_index((0.5, 23.5), center, coords, types, radii, 28)
+        lib.mg_forward_index_paged(0)
+        close(plain, ref, name + " forward")
+        close(paged, plain, name + " paged write-out", exact=True)
+        rng = np.random.default_rng(5)
+        diff = rng.standard_normal(ref.shape).astype(np.float32)
+        ref32 = og.backward(center, coords, types, radii, diff)
+        ref64 = og.backward(center, coords, types, radii, diff, f64=True)
+        mag = np.abs(og.backward(center, coords, types, radii, np.abs(diff), f64=True)).max(
+            axis=1, keepdims=True) + 1e-30
+        g = E.gridmaker(0.5, 23.5)
+        n = len(coords)
+        grads = E.array((n, 3), fill=9.0)
+        assert lib.mg_backward_index(ctypes.byref(g), 1, None, n, None, E.f3(center),
+                                     E.ptr(E.put(coords)), E.ptr(E.put(types)), E.ptr(E.put(radii)), 28,
+                                     E.ptr(E.put(diff)), E.ptr(grads), None) == 0
+        check_grads(grads, ref32, ref64, mag, name + " backward")
+
+
 GROUPS = {k[len("group_"):]: v for k, v in list(globals().items()) if k.startswith("group_")}
 
 if __name__ == "__main__":

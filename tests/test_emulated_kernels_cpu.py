@@ -25,7 +25,8 @@ def emulated_library():
 
 
 @pytest.mark.parametrize("group", ["transform", "forward_index", "forward_batch", "forward_paged", "forward_split", "backward_index",
-                                   "forward_vector", "backward_vector", "second_order", "interpolate"])
+                                   "forward_vector", "backward_vector", "second_order", "interpolate",
+                                   "config0"])
 def test_group(emulated_library, group):
     p = subprocess.run([sys.executable, RUNNER, group], stdout=subprocess.PIPE,
                        stderr=subprocess.STDOUT, text=True, timeout=1200)
