@@ -282,53 +282,3 @@ def test_more_atoms_than_sixteen_bit_indices(mg):
             assert_close(got, ref, what="70,000 atoms")
     assert ref.sum() > 100
 
-
-@pytest.mark.parametrize("binary", [False, True])
-def test_sort_and_splat_on_two_streams_equal_forward_batch(mg, binary):
-    """mg_forward_index_sort on a side stream, mg_forward_index_splat on the main one after an
-    event: the grids of forward_batch, bit for bit."""
-    c = synth.config1(nbatch=6)
-    gm = mg.GridMaker(0.5, 23.5, binary)
-    batch = mg.AtomBatch(c["offsets"])
-    coords, types, radii, centers = [dev(c[k]) for k in ("coords", "types", "radii", "centers")]
-    whole = torch.full((6,) + gm.grid_dimensions(28), 7.0, device="cuda")
-    gm.forward_batch(batch, centers, coords, types, radii, whole)
-    split = torch.full_like(whole, 7.0)
-    side, main = torch.cuda.Stream(), torch.cuda.current_stream()
-    ready, sorted_done = torch.cuda.Event(), torch.cuda.Event()
-    ready.record(main)
-    side.wait_event(ready)
-    with torch.cuda.stream(side):
-        sb = gm.sort_batch(batch, centers, coords, types, radii, 28)
-        sorted_done.record(side)
-    main.wait_event(sorted_done)
-    gm.splat_batch(sb, split)
-    torch.cuda.synchronize()
-    assert torch.equal(split, whole)
-    with pytest.raises(ValueError):
-        gm.splat_batch(sb, torch.empty((5,) + gm.grid_dimensions(28), device="cuda"))
-
-
-@pytest.mark.parametrize("binary", [False, True])
-@pytest.mark.parametrize("res,dimension,ntypes,natoms", [
-    (0.5, 23.5, 28, 300), (1.0, 15.0, 40, 200), (0.25, 5.75, 2, 15), (0.5, 3.5, 3, 12)])
-def test_paged_write_out_gives_the_same_grids(mg, res, dimension, ntypes, natoms, binary):
-    """The write-out in whole 4 KB pages (mg_forward_index_paged) against the per-wave one, bit for
-    bit, and against the oracle."""
-    from libmolgrid_amd import _capi
-    rng = np.random.default_rng(31 + natoms)
-    coords, types, radii = synth.small_index_case(rng, natoms, ntypes, dimension / 2 + 2.0)
-    center = rng.uniform(-1, 1, 3).astype(np.float32)
-    ref = oracle.GridMaker(res, dimension, binary).forward(center, coords, types, radii, ntypes)
-    before = _capi.lib.mg_forward_index_paged(0)
-    try:
-        plain = gpu_forward(mg, (res, dimension, binary), center, coords, types, radii, ntypes)
-        _capi.lib.mg_forward_index_paged(1)
-        paged = gpu_forward(mg, (res, dimension, binary), center, coords, types, radii, ntypes)
-    finally:
-        _capi.lib.mg_forward_index_paged(before)
-    assert np.array_equal(paged, plain)
-    if binary:
-        assert np.array_equal(paged, ref)
-    else:
-        assert_close(paged, ref, what="paged forward")

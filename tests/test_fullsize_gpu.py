@@ -53,29 +53,6 @@ def test_forward_every_example(mg, workload):
         assert torch.equal(one, out[b])
 
 
-@pytest.mark.parametrize("binary", [False, True])
-def test_paged_write_out_full_batch(mg, workload, binary):
-    """The whole benchmark batch through the write-out in 4 KB pages: the grids of the per-wave
-    write-out, bit for bit (which test_forward_every_example holds against the oracle)."""
-    from libmolgrid_amd import _capi
-    c = workload
-    B = len(c["offsets"]) - 1
-    gm = mg.GridMaker(0.5, 23.5, binary)
-    batch = mg.AtomBatch(c["offsets"])
-    moved, types, radii, centers = dev(c["moved"]), dev(c["types"]), dev(c["radii"]), dev(c["centers"])
-    plain = torch.full((B,) + gm.grid_dimensions(28), -1.0, device="cuda")
-    paged = torch.full_like(plain, -2.0)
-    before = _capi.lib.mg_forward_index_paged(0)
-    try:
-        gm.forward_batch(batch, centers, moved, types, radii, plain)
-        _capi.lib.mg_forward_index_paged(1)
-        gm.forward_batch(batch, centers, moved, types, radii, paged)
-    finally:
-        _capi.lib.mg_forward_index_paged(before)
-    torch.cuda.synchronize()
-    assert torch.equal(paged, plain)
-
-
 def test_binary_grid_ignores_atom_order(mg, workload):
     c = workload
     B = len(c["offsets"]) - 1

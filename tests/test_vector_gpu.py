@@ -167,31 +167,3 @@ def test_type_gradient_is_density_dot_diff(mg):
         want = (one[0][None] * diff).sum(dim=(1, 2, 3)).cpu().numpy()
         np.testing.assert_allclose(tg[a].cpu().numpy(), want, rtol=1e-4, atol=1e-4)
 
-
-@pytest.mark.parametrize("binary", [False, True])
-def test_atom_lists_give_the_same_grids(mg, binary):
-    """mg_forward_vector_ws with its workspace (a launch before the splat lists the atoms that can
-    reach each slab of four x planes) against mg_forward_vector without: bit for bit, on a ragged
-    batch at the benchmark's resolution."""
-    import ctypes
-    from libmolgrid_amd import _capi
-    v = synth.vector_batch(nbatch=3, natoms=1200)
-    gm = mg.GridMaker(0.25, 23.75, binary)
-    off = torch.as_tensor(v["offsets"].astype(np.int32)).cuda()
-    cen, c, t, r = [dev(v[k]) for k in ("centers", "coords", "types", "radii")]
-    shape = (3,) + gm.grid_dimensions(28)
-    plain = torch.full(shape, 5.0, device="cuda")
-    listed = torch.full(shape, 6.0, device="cuda")
-    args = [gm._p, 3, off.data_ptr(), 1200, cen.data_ptr(), _capi.f3((0, 0, 0)), c.data_ptr(),
-            t.data_ptr(), r.data_ptr(), 28]
-    assert _capi.lib.mg_forward_vector(*args, plain.data_ptr(), None) == 0
-    need = int(_capi.lib.mg_forward_vector_workspace_size(gm._p, 3, 1200, 28))
-    assert need > 0
-    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-    assert _capi.lib.mg_forward_vector_ws(*args, listed.data_ptr(), ws.data_ptr(), need, None) == 0
-    torch.cuda.synchronize()
-    assert torch.equal(listed, plain)
-    # the Python layer takes the workspace path
-    out = torch.full(shape, 7.0, device="cuda")
-    gm.forward_batch(v["offsets"], cen, c, t, r, out)
-    assert torch.equal(out, plain)
