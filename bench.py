@@ -2,7 +2,7 @@
 """Benchmark of the gridding hot path on one MI355X.
 
 A step is one pass over one synthetic batch of 50 ragged complexes
-(configuration 1/2 of BASELINE.json): per-example rigid transform of the atoms,
+(configurations 1 and 2 of the benchmark definition): per-example rigid transform of the atoms,
 forward splat into a 50x28x48^3 float32 tensor, atom-gradient backward against a
 N(0,1) upstream gradient and the un-rotation of those gradients.  All inputs are
 resident in HBM before the timed region.  One JSON line is printed.

@@ -523,7 +523,7 @@ def group_interpolate():
 
 
 def group_config0():
-    """BASELINE configuration 0 at full size (1,540 atoms into 28 x 48^3) plus one example of
+    """The benchmark's configuration 0 at full size (1,540 atoms into 28 x 48^3) plus one example of
     configuration 1 (rotated, translated): forward in both write-outs, backward."""
     lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
     c0 = synth.config0()
