@@ -354,7 +354,7 @@ template <bool BINARY, bool EXACT, int COLS, bool PAGED>
 __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sorted_kernel(
     GridArg g, const float4* __restrict__ slot_info, const int* __restrict__ cand,
     const float4* __restrict__ records, int capacity, float* __restrict__ out,
-    int nxs, int nyp, int nzs, int nranges, int aligned_rows, int slab_z) {
+    int nxs, int nyp, int nzs, int nranges, int aligned_rows, int slab_z, int nbatch) {
   // one column of one wave (rows padded), or the workgroup's slab of four x planes
   __shared__ __align__(16) float stage[PAGED ? kSlabFloats : kPlane];
 
@@ -415,13 +415,17 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
   if (nmine <= 0) return;
 
   const float4 info = slot_info[slot];
-  const int e = __builtin_amdgcn_readfirstlane(__float_as_int(info.w));
+  // (what comes out of the workspace is held inside its bounds, so that a workspace that the sort
+  // launch did not fill for these sizes gives wrong grids, not a fault or an endless loop)
+  const int e = min(max(__builtin_amdgcn_readfirstlane(__float_as_int(info.w)), 0), nbatch - 1);
   // first and one-past-last candidate record of this lane's channel
   const __amdgpu_buffer_rsrc_t cand_buf =
       buffer_of(cand + (size_t)slot * ntypes * nxs * 2, (size_t)ntypes * nxs * 8);
   const int my_chan = range + lane * nranges;
   v2u se = {0u, 0u};
   if (lane < nmine) se = __builtin_amdgcn_raw_buffer_load_b64(cand_buf, (my_chan * nxs + xs) * 8, 0, 0);
+  se.x = min(se.x, (unsigned)capacity);
+  se.y = min(se.y, (unsigned)capacity);
 
   const int x0 = xs * kColXY, y0 = yp * (kColXY * COLS), z0 = zs * slab_z;
   const int zend = min(z0 + slab_z, dim);
@@ -745,7 +749,7 @@ hipError_t launch_splat_paged(const GridArg& g, const SortedAtoms& s, int nbatch
   if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
   hipLaunchKernelGGL((splat_sorted_kernel<BINARY, false, 2, true>), dim3((unsigned)nitems),
                      dim3(nyp * kWave), 0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out,
-                     nxs, nyp, 1, g.ntypes, 1, kSlabZ);
+                     nxs, nyp, 1, g.ntypes, 1, kSlabZ, nbatch);
   return hipGetLastError();
 }
 
@@ -768,7 +772,7 @@ hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, floa
   const int aligned = ((dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
   hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS, false>), dim3((unsigned)nitems), dim3(kWave),
                      0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out, nxs, nyp, nzs,
-                     nranges, aligned, slab_z);
+                     nranges, aligned, slab_z, nbatch);
   return hipGetLastError();
 }
 

@@ -193,6 +193,16 @@ def group_forward_split():
         assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(ws), need,
                                           None) == 0
         close(out, whole, "sort + splat, binary=%s" % binary, exact=True)
+    # a workspace the sort launch never filled (0xCB bytes, then random bytes): wrong grids are
+    # fine, leaving the arrays or looping for ever is not
+    junk = E.array(need, np.uint8, tight=False)
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(junk), need, None) == 0
+    junk[...] = np.random.default_rng(1).integers(0, 256, need, dtype=np.uint8)
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(junk), need, None) == 0
+    lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    lib.mg_forward_index_paged(1)
+    assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(junk), need, None) == 0
+    lib.mg_forward_index_paged(0)
     # argument errors: a workspace that is too small or misaligned, no workspace
     assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), E.ptr(ws), need - 1, None) == -1
     assert lib.mg_forward_index_splat(ctypes.byref(g), 5, width, 6, E.ptr(out), ws[16:].ctypes.data, need, None) == -1
