@@ -37,6 +37,9 @@ def build(verbose=True):
     objs = []
     for src, obj, p in procs:
         out, _ = p.communicate()
+        # hipcc compiles every source twice, for gfx950 and for the host; the flag above names a
+        # gfx950 feature, the device pass honours it (no v_pk_*_f32 in the ISA) and the HOST pass
+        # (x86-64) says it does not know the feature -- that one line is dropped here
         out = "\n".join(l for l in out.splitlines()
                         if "packed-fp32-ops' is not a recognized feature" not in l)
         if p.returncode != 0:
