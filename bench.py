@@ -150,7 +150,7 @@ def parity_sample(cfg, gm_args, ntypes, nsample, moved, grid, diff, grads):
 
 
 def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, diff, grads,
-                    n_atoms, bwd_bytes):
+                    n_atoms, bwd_bytes, small=False):
     """The remaining configurations, one kernel each, events on the launch stream: the backward
     pass with 90 % of the upstream gradient zeroed (configuration 2), vector types into 28x96^3
     for Gaussian and binary density (configuration 3), trilinear resampling under random rotations
@@ -192,32 +192,33 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
                                         "random rotation, +-1.5 A" % (B, K, D))
 
     # configuration 3: 16 x 10,000 atoms with 28-float type vectors into 28x96^3
-    v = synth.vector_batch(nbatch=16, natoms=10000)
+    VB, VN = (2, 300) if small else (16, 10000)    # small: a dry run of this function, not a figure
+    v = synth.vector_batch(nbatch=VB, natoms=VN)
     ab = mg.AtomBatch(v["offsets"])
     ab.dev
     vc, vt, vr = [torch.as_tensor(v[k]).cuda() for k in ("coords", "types", "radii")]
     vcen = torch.as_tensor(v["centers"]).cuda()
     for binary in (False, True):
         gv = mg.GridMaker(0.25, 23.75, binary)
-        out = torch.empty((16,) + gv.grid_dimensions(28), device="cuda")
+        out = torch.empty((VB,) + gv.grid_dimensions(28), device="cuda")
         ms = event_ms(lambda: gv.forward_batch(ab, vcen, vc, vt, vr, out), 5)
         nbytes = out.numel() * 4 + vc.shape[0] * (16 + 4 * 28)
         res["forward_vector_binary" if binary else "forward_vector"] = entry(
-            ms, nbytes, grids_per_s=round(16 / (ms * 1e-3), 1),
-            workload="configs[3]: 16 x 10,000 atoms, 28x96^3 at 0.25 A")
+            ms, nbytes, grids_per_s=round(VB / (ms * 1e-3), 1),
+            workload="configs[3]: %d x %d atoms, 28x96^3 at 0.25 A" % (VB, VN))
         del out
     try:
         # backward pass for vector types on the same atoms (atom and type gradients): the upstream
         # gradient 16 x 28 x 96^3 is read once
         gv = mg.GridMaker(0.25, 23.75)
-        vdiff = torch.randn((16,) + gv.grid_dimensions(28), device="cuda",
+        vdiff = torch.randn((VB,) + gv.grid_dimensions(28), device="cuda",
                             generator=torch.Generator(device="cuda").manual_seed(3))
         vag, vtg = torch.empty_like(vc), torch.empty_like(vt)
         ms = event_ms(lambda: gv.backward_batch(ab, vcen, vc, vt, vr, vdiff, vag, vtg), 3, warmup=1)
         res["backward_vector"] = entry(
             ms, vdiff.numel() * 4 + vc.shape[0] * (16 + 4 * 28) + vc.shape[0] * (12 + 4 * 28),
             atom_grads_per_s=round(vc.shape[0] / (ms * 1e-3), 1),
-            workload="configs[3] atoms: atom + type gradients against a N(0,1) gradient 16x28x96^3")
+            workload="configs[3] atoms: atom + type gradients against a N(0,1) gradient %dx28x96^3" % VB)
         del vdiff, vag, vtg
     except Exception as e:          # a new measurement must not cost the bench line
         res["backward_vector"] = {"error": repr(e)[:200]}
@@ -257,12 +258,12 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
     # the same atoms with radii by type instead of by atom (a density per atom AND channel: no
     # matrix product, 28 times the density evaluations)
     gv = mg.GridMaker(0.25, 23.75, False, True)
-    tr = torch.as_tensor(np.random.default_rng(11).uniform(1.2, 2.0, (16, 28)).astype(np.float32)).cuda()
-    out = torch.empty((16,) + gv.grid_dimensions(28), device="cuda")
+    tr = torch.as_tensor(np.random.default_rng(11).uniform(1.2, 2.0, (VB, 28)).astype(np.float32)).cuda()
+    out = torch.empty((VB,) + gv.grid_dimensions(28), device="cuda")
     ms = event_ms(lambda: gv.forward_batch(ab, vcen, vc, vt, tr, out), 3, warmup=1)
     res["forward_vector_type_radii"] = entry(
-        ms, out.numel() * 4 + vc.shape[0] * (12 + 4 * 28), grids_per_s=round(16 / (ms * 1e-3), 1),
-        workload="configs[3] atoms with type-indexed radii (16 x 28 radii), Gaussian")
+        ms, out.numel() * 4 + vc.shape[0] * (12 + 4 * 28), grids_per_s=round(VB / (ms * 1e-3), 1),
+        workload="configs[3] atoms with type-indexed radii (%d x 28 radii), Gaussian" % VB)
     del out
     return res
 
@@ -281,6 +282,9 @@ def main():
                     help="skip the forward call with every atom ignored (the write stream alone) "
                          "and the plain fill: for profiling runs, whose per-kernel means then "
                          "cover the real calls only")
+    ap.add_argument("--small-extras", action="store_true",
+                    help="cut the vector-type workloads down to 2 x 300 atoms: for dry runs of this "
+                         "script (an emulated device), not for figures")
     ap.add_argument("--no-graph", action="store_true",
                     help="do not time the step as a captured HIP graph")
     ap.add_argument("--serial-only", action="store_true",
@@ -535,7 +539,7 @@ def main():
 
     if not args.no_extras:
         kernels.update(other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid,
-                                       diff, grads, n_atoms, bwd_bytes))
+                                       diff, grads, n_atoms, bwd_bytes, small=args.small_extras))
 
     cpu = None
     if not args.no_cpu:

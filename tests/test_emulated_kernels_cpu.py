@@ -43,3 +43,27 @@ def test_hostile_inputs_return(emulated_library):
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
     assert p.returncode == 0, "fuzz failed (status %d):\n%s" % (p.returncode, p.stdout[-3000:])
     assert "12 rounds returned" in p.stdout
+
+
+def _run(script, *flags, timeout=2400):
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", script)] + list(flags),
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+    assert p.returncode == 0, "%s failed (status %d):\n%s" % (script, p.returncode, p.stdout[-4000:])
+    return p.stdout
+
+
+def test_python_host_layer_on_a_fake_device(emulated_library):
+    """tests/emu/python_layer.py: GridMaker / Transform / GridInterpolater / Coords2Grid of the
+    package on a stand-in for the ROCm device (CPU tensors that say they are on cuda:0, the emulated
+    kernels behind the C ABI) against the oracle: forward overloads, workspaces, the sort and splat
+    halves, backward with the fused un-rotation, vector types with atom lists, autograd, resampling."""
+    assert "comparisons passed" in _run("python_layer.py")
+
+
+def test_smoke_and_bench_run_end_to_end_on_a_fake_device(emulated_library):
+    """__graft_entry__.smoke() and bench.py (a batch of one example, every step variant, the
+    write-out autotune, the JSON line with the fields the driver reads) on the same stand-in: the
+    figures mean nothing, the code paths are what is checked.  The other workloads of bench.py are
+    left out here (tests/emu/bench_dry_run.py --small-extras by hand runs them too, minutes)."""
+    assert "passed" in _run("smoke_dry_run.py")
+    assert "JSON line complete" in _run("bench_dry_run.py", "--no-extras", "--no-cpu")
