@@ -150,7 +150,12 @@ def activate():
     torch.cuda.CUDAGraph = _NoGraph
     torch.cuda.graph = _NoGraph
     real_generator = torch.Generator
-    torch.Generator = lambda device=None: real_generator()
+
+    class HostGenerator(real_generator):              # a generator "on the device" is a host one
+        def __new__(cls, device=None):
+            return real_generator.__new__(cls)
+
+    torch.Generator = HostGenerator
     for name in ("empty", "zeros", "ones", "full", "randn", "rand", "arange", "tensor"):
         setattr(torch, name, _factory(getattr(torch, name)))
     real_as_tensor = torch.as_tensor
@@ -162,9 +167,10 @@ def activate():
     def to(self, *a, **k):
         dev = k.get("device", a[0] if a and not isinstance(a[0], torch.dtype) else None)
         if _is_cuda_device(dev):
-            k.pop("device", None)
-            a = tuple(x for x in a if x is not dev)
-            moved = real_to(self, *a, **k) if (a or k) else self
+            if "device" in k:
+                k["device"] = "cpu"
+            a = tuple("cpu" if x is dev else x for x in a)
+            moved = real_to(self, *a, **k)
             return moved if isinstance(self, DevTensor) and moved is self else on_device(
                 moved.clone() if moved.data_ptr() == self.data_ptr() else moved)
         return real_to(self, *a, **k)
