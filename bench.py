@@ -482,6 +482,17 @@ def main():
     if not args.no_write_stream:
         types_none = torch.full_like(types, -1.0)
         ms_fwd_stores = event_ms(lambda: gm.forward_batch(offsets, centers, moved, types_none, radii, grid), it)
+        # ... and in the write-out that is not in use, whose store skeleton is the other shape
+        # (per wave: row groups of 768 bytes; paged: whole 4 KB pages from workgroups of six waves)
+        other_stores = None
+        try:
+            from libmolgrid_amd import _capi
+            was = _capi.lib.mg_forward_index_paged(0)
+            _capi.lib.mg_forward_index_paged(0 if was else 1)
+            other_stores = event_ms(lambda: gm.forward_batch(offsets, centers, moved, types_none, radii, grid), it)
+            _capi.lib.mg_forward_index_paged(was)
+        except Exception:
+            pass
         ms_fill = event_ms(lambda: grid.zero_(), it)
         del types_none
         k_forward()                               # the grids of the step again
@@ -510,6 +521,8 @@ def main():
         "write_stream_alone": None if ms_fwd_stores is None else {
             "forward_call_all_atoms_ignored_ms": round(ms_fwd_stores, 4),
             "frac": round(fwd_bytes / (ms_fwd_stores * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "write_out": (write_out or {}).get("used", "per_wave"),
+            "other_write_out_ms": None if other_stores is None else round(other_stores, 4),
             "torch_fill_ms": round(ms_fill, 4),
             "torch_fill_frac": round(grid_bytes / (ms_fill * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         # the same kernel between the other launches of the step (see step_breakdown)
