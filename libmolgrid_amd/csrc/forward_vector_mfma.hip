@@ -118,7 +118,7 @@ splat_vector_mfma_kernel(
   float vx[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t)
-    vx[t] = x0 + t < dim ? grid_coord(ox, x0 + t, g.resolution) : INFINITY;   // outside: unreachable
+    vx[t] = uniform(x0 + t < dim ? grid_coord(ox, x0 + t, g.resolution) : INFINITY);   // outside: unreachable
 
   const float clx = uniform(grid_coord(ox, x0, g.resolution));
   const float clz = uniform(grid_coord(oz, z0, g.resolution));
@@ -398,10 +398,14 @@ splat_vector_mfma_kernel(
       // takes the registers e = 2p and 2p + 1 of the tiles of one h: every lane writes two
       // channels, plane 2 * quad + (e & 1) of the stage holds channel
       // 16 * h + 4 * quad + 2 * p + (e & 1).
+      // (worked out here, after the steps, and not once before them, where these nine values
+      // would sit in scratch memory for the whole column)
       int st_lds[kPer], st_slot[kPer], st_sp[kPer];
+      int tid_now = tid;
+      compute_here(tid_now);
 #pragma unroll
       for (int k = 0; k < kPer; ++k) {
-        const int item = tid + k * kColThreads;
+        const int item = tid_now + k * kColThreads;
         const int jj = item / 192, q = item % 192, row = q / 12, f4 = q % 12;
         const int gx = x0 + (row >> 2), gy = y0 + (row & 3), gz = z0 + f4 * 4;
         st_lds[k] = jj * kPlaneS + row * kRowPad + f4 * 4;

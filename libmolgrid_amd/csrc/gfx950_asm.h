@@ -16,6 +16,11 @@ __device__ __forceinline__ float mul_legacy(float a, float b) {
 // keeps a wave-uniform value in a vector register (an fma takes one scalar operand)
 __device__ __forceinline__ void keep_in_vgpr(float& v) { asm volatile("" : "+v"(v)); }
 
+// The same for an integer, used the other way round: what is computed from the value after this
+// point cannot be moved in front of it (out of a loop, where it would occupy registers -- or
+// scratch memory -- for the whole loop).
+__device__ __forceinline__ void compute_here(int& v) { asm volatile("" : "+v"(v)); }
+
 // workgroup barrier that waits for the wave's LDS traffic only (not for its global loads and
 // stores, which __syncthreads would also wait for)
 __device__ __forceinline__ void lds_barrier() {

@@ -260,6 +260,7 @@ namespace mg {
 inline float mul_legacy(float a, float b) { return (a == 0.f || b == 0.f) ? 0.f : a * b; }
 inline void keep_in_vgpr(float&) {}
 inline void keep_branch() {}
+inline void compute_here(int&) {}
 inline void lds_barrier() { emu::barrier(); }
 // the lanes of a wave are fibers here and do not run in step: meet
 inline void wave_lds_fence() { uint64_t live; (void)emu::gather(0, &live, "wave_lds_fence"); }
