@@ -350,6 +350,17 @@ __global__ __launch_bounds__(kSortThreads) void sort_atoms_kernel(
 // ------------------------------------------------------------------------------------------
 // Launch 2
 // ------------------------------------------------------------------------------------------
+// Last block at or below `top` and first block at or above `bottom` of a column's blocks
+// 0 .. last: -1 and last + 1 when there is none.  The clamps are float operations, so that the
+// conversion never sees a value outside the range of int (fminf and fmaxf return the other
+// operand for not-a-number: a record with such a coordinate selects every block of the column).
+__device__ __forceinline__ int block_below(float top, int last) {
+  return (int)fmaxf(fminf(floorf(top), (float)last), -1.f);
+}
+__device__ __forceinline__ int block_above(float bottom) {
+  return (int)fminf(fmaxf(ceilf(bottom), 0.f), 32.f);
+}
+
 template <bool BINARY, bool EXACT, int COLS, bool PAGED>
 __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sorted_kernel(
     GridArg g, const float4* __restrict__ slot_info, const int* __restrict__ cand,
@@ -593,7 +604,9 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
           // block q holds the voxel centres clz + (4q .. 4q+3) * resolution
           const float top = (rec_z + rz - clz) * inv_block + 1e-3f;
           const float bottom = (rec_z - rz - clz) * inv_block - (0.75f + 1e-3f);
-          const int qhi = min((int)floorf(top), last_block), qlo = max((int)ceilf(bottom), 0);
+          // (clamped as floats, so that no record -- huge, infinite, not a number -- reaches the
+          // conversion out of range)
+          const int qhi = block_below(top, last_block), qlo = block_above(bottom);
           if (qlo <= qhi) mask[col] = (2u << qhi) - (1u << qlo);
           if (!BINARY && !EXACT) {
             // bits 16..27: the blocks that the Gaussian core of the atom (u <= grm^2) can reach,
@@ -603,7 +616,7 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
               const float cz = __builtin_amdgcn_sqrtf(cz2);
               const float ctop = (rec_z + cz - clz) * inv_block + 1e-3f;
               const float cbottom = (rec_z - cz - clz) * inv_block - (0.75f + 1e-3f);
-              const int chi = min((int)floorf(ctop), last_block), clo = max((int)ceilf(cbottom), 0);
+              const int chi = block_below(ctop, last_block), clo = block_above(cbottom);
               if (clo <= chi) mask[col] |= (((2u << chi) - (1u << clo)) & mask[col]) << 16;
             }
           }

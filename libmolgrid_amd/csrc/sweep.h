@@ -123,8 +123,10 @@ __device__ __forceinline__ void sweep_channel(const GridArg& g, const float* __r
 __device__ __forceinline__ void reach_range(float origin, float coord, float reach, float inv_res,
                                             int dim, int& lo, int& n) {
   constexpr float kSlack = 1e-3f;
-  const float first = fmaxf(ceilf((coord - reach - origin) * inv_res - kSlack), 0.f);
-  const float last = fminf(floorf((coord + reach - origin) * inv_res + kSlack), (float)(dim - 1));
+  // (clamped on both sides as floats: a coordinate or a reach that is huge, infinite or not a
+  // number must not reach the conversion)
+  const float first = fminf(fmaxf(ceilf((coord - reach - origin) * inv_res - kSlack), 0.f), (float)dim);
+  const float last = fmaxf(fminf(floorf((coord + reach - origin) * inv_res + kSlack), (float)(dim - 1)), -1.f);
   lo = (int)first;
   n = (int)last - lo + 1;
 }

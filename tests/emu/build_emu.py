@@ -8,9 +8,26 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "libmolgrid_amd", "csrc")
-LIB_PATH = os.path.join(HERE, "libmolgrid_emu.so")
 SOURCES = ["capi.hip", "transform.hip", "convert.hip", "forward_sorted.hip", "forward_vector.hip",
            "forward_vector_mfma.hip", "backward.hip", "second_order.hip", "interpolate.hip"]
+
+# EMU_SANITIZE selects a second build of the same sources with clang's run-time checks, every report
+# fatal: "1" the undefined-behaviour checks (array indices of fixed-size arrays -- the register and
+# LDS arrays of the kernels --, shifts, signed overflow, float-to-int conversions out of range,
+# misaligned accesses), "list" the same but reporting and going on (to see every place at once),
+# "address" the address checks (every LDS array -- static storage here -- and every stack array gets
+# poisoned neighbours, so an access through a pointer that leaves its array is caught as well).
+SANITIZE = os.environ.get("EMU_SANITIZE", "")
+if SANITIZE in ("0",):
+    SANITIZE = ""
+if SANITIZE == "address":
+    SAN_FLAGS = ["-fsanitize=address", "-fno-omit-frame-pointer"]
+    TAG = "asan"
+else:
+    SAN_FLAGS = ["-fsanitize=undefined,float-cast-overflow", "-fno-sanitize=vptr,function",
+                 "-fsanitize-recover=all" if SANITIZE == "list" else "-fno-sanitize-recover=all"]
+    TAG = "ubsan"
+LIB_PATH = os.path.join(HERE, "libmolgrid_emu_%s.so" % TAG if SANITIZE else "libmolgrid_emu.so")
 
 
 def _compiler():
@@ -35,11 +52,13 @@ def build(force=False, verbose=False):
     if not force and up_to_date():
         return LIB_PATH
     cxx = _compiler()
-    objdir = os.path.join(HERE, "build")
+    objdir = os.path.join(HERE, "build_" + TAG if SANITIZE else "build")
     os.makedirs(objdir, exist_ok=True)
     flags = ["-std=c++17", "-O1", "-g", "-fPIC", "-ffp-contract=off", "-Wno-unknown-attributes",
              "-Wno-ignored-attributes", "-Wno-unused-value", "-Wno-pass-failed",
              "-I" + HERE, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    if SANITIZE:
+        flags += SAN_FLAGS
     procs = []
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
@@ -58,7 +77,11 @@ def build(force=False, verbose=False):
         if verbose and out.strip():
             print(out)
         objs.append(obj)
-    subprocess.check_call([cxx, "-shared", "-fPIC"] + objs + ["-o", LIB_PATH])
+    link = []
+    if SANITIZE:      # the checks' runtime as a shared library, found beside the compiler
+        rt = subprocess.check_output([cxx, "-print-resource-dir"], text=True).strip() + "/lib/linux"
+        link = SAN_FLAGS + ["-shared-libsan", "-Wl,-rpath," + rt]
+    subprocess.check_call([cxx, "-shared", "-fPIC"] + link + objs + ["-o", LIB_PATH])
     return LIB_PATH
 
 

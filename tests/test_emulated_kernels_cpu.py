@@ -45,6 +45,26 @@ def test_hostile_inputs_return(emulated_library):
     assert "12 rounds returned" in p.stdout
 
 
+@pytest.mark.parametrize("checks", ["undefined", "address"])
+def test_run_time_checks(emulated_library, checks):
+    """The same sources built again with clang's run-time checks, every report fatal, running the
+    comparison groups of the kernels and a few rounds of hostile inputs.  "undefined": fixed-size
+    array indices (the register and LDS arrays), shifts, signed overflow, float-to-int conversions
+    out of range, alignment -- a conversion of an infinite coordinate is what these found.
+    "address": every LDS array (static storage in the emulation) and stack array has poisoned
+    neighbours, so an access through a pointer that leaves its array is caught too (the runtime is
+    loaded with the library, after the interpreter: hence verify_asan_link_order=0)."""
+    env = dict(os.environ, EMU_SANITIZE="1" if checks == "undefined" else "address",
+               ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
+    for args in (["cases.py", "forward_index"], ["cases.py", "forward_paged"], ["cases.py", "backward_index"],
+                 ["cases.py", "forward_vector"], ["cases.py", "backward_vector"], ["cases.py", "second_order"],
+                 ["cases.py", "interpolate"], ["fuzz.py", "8", "5"]):
+        p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+        assert p.returncode == 0 and "runtime error" not in p.stdout and "AddressSanitizer" not in p.stdout, \
+            "%s under the %s checks (status %d):\n%s" % (" ".join(args), checks, p.returncode, p.stdout[-3000:])
+
+
 def _run(script, *flags, timeout=2400):
     p = subprocess.run([sys.executable, os.path.join(HERE, "emu", script)] + list(flags),
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
