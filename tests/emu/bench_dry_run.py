@@ -20,6 +20,11 @@ import fake_cuda  # noqa: E402
 fake_cuda.activate()
 import bench  # noqa: E402
 
+if "--candidates" in sys.argv:          # started by bench.py itself: its child process, same device
+    sys.argv = ["bench.py"] + sys.argv[1:]
+    bench.main()
+    sys.exit(0)
+bench.CANDIDATE_COMMAND = [sys.executable, os.path.abspath(__file__)]
 sys.argv = ["bench.py", "--batch", "1", "--steps", "1", "--warmup", "0"] + sys.argv[1:]
 buf = io.StringIO()
 with redirect_stdout(buf):
