@@ -23,7 +23,10 @@ __global__ __launch_bounds__(kSplatThreads) void splat_vector_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_vector, const float* __restrict__ radii,
     float* __restrict__ out, int tiles_per_side, int vec_store) {
-  HIP_DYNAMIC_SHARED(float, s_stage);               // [TG][512], output staging (16-byte aligned)
+  // [TG][512] floats of output staging, declared as 16-byte vectors so that the compiler knows
+  // the alignment (the write-out reads it with one 128-bit LDS instruction per piece)
+  HIP_DYNAMIC_SHARED(v4f, s_stage_v4);
+  float* const s_stage = reinterpret_cast<float*>(s_stage_v4);
   __shared__ int s_cand[kCandCap];
   __shared__ float4 s_rec[kChunk];   // x, y, z, (ar^2 | 1/ar^2) (w unused when RTI)
   __shared__ int s_recatom[kChunk];  // atom index of each record
