@@ -488,25 +488,35 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
     const unsigned lead = (unsigned)((reinterpret_cast<uintptr_t>(chan) + first) & (kPageBytes - 1));
     const int npages = (int)((lead + bytes + kPageBytes - 1) / kPageBytes);
     const float inv_pieces = 4.0f / (float)dim, inv_dim = 1.0f / (float)dim;
-    const int prow = paged_row(dim), pplane = paged_plane(dim);
+    // the slab in 16-byte pieces (rows and planes are whole pieces: dim % 4 == 0)
+    const v4f* const slab = reinterpret_cast<const v4f*>(stage);
+    const int prow4 = paged_row(dim) >> 2, pplane4 = paged_plane(dim) >> 2, dim4 = dim >> 2;
+    const unsigned dropped = (unsigned)(chan_stride * 4);               // an offset past the channel
+    constexpr int kStores = kPageBytes / (kWave * 16);                  // 4 stores of 1 KB a page
     for (int page = (int)(threadIdx.x >> 6); page < npages; page += (int)(blockDim.x >> 6)) {
+      // All four pieces are read from LDS first and then stored by four instructions in a row,
+      // none of them in a branch: the memory system takes a page fastest as one burst.  A piece
+      // before the slab's first byte or after its last (a page shared with the neighbouring slab)
+      // is stored to an offset past the end of the channel, which the hardware drops.
+      unsigned off[kStores];
+      v4f v[kStores];
 #pragma unroll
-      for (int k = 0; k < kPageBytes / (kWave * 16); ++k) {
+      for (int k = 0; k < kStores; ++k) {
         // byte of this lane's piece relative to the slab's start
         const int rel = page * kPageBytes + (k * kWave + lane) * 16 - (int)lead;
-        if (rel >= 0 && rel < (int)bytes) {
-          v4f v = {0.f, 0.f, 0.f, 0.f};
-          if (from_slab) {
-            const int piece = rel >> 4;
-            const int row = (int)(((float)piece + 0.5f) * inv_pieces);   // piece / (dim / 4)
-            const int px = (int)(((float)row + 0.5f) * inv_dim);         // row / dim
-            v = *reinterpret_cast<const v4f*>(stage + px * pplane + (row - px * dim) * prow +
-                                              (piece * 4 - row * dim));
-          }
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), out_buf,
-                                                 (int)(first + (unsigned)rel), 0, 2);
+        const bool mine = rel >= 0 && rel < (int)bytes;
+        off[k] = mine ? first + (unsigned)rel : dropped;
+        v[k] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (from_slab) {
+          const int piece = mine ? rel >> 4 : 0;
+          const int row = (int)(((float)piece + 0.5f) * inv_pieces);     // piece / (dim / 4)
+          const int px = (int)(((float)row + 0.5f) * inv_dim);           // row / dim
+          v[k] = slab[px * pplane4 + (row - px * dim) * prow4 + (piece - row * dim4)];
         }
       }
+#pragma unroll
+      for (int k = 0; k < kStores; ++k)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v[k]), out_buf, (int)off[k], 0, 2);
     }
   };
 
