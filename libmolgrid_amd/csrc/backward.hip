@@ -56,10 +56,27 @@ __device__ __forceinline__ float grad_scale(const GradConsts& c, float dist2, fl
   return (dist2 <= c.reach2) ? s * gridval : 0.f;
 }
 
-template <bool BINARY>
+// The same for a Gaussian that is cut off without a tail (final radius multiple = Gaussian
+// multiple): there the scale jumps at the cut-off, so whether a voxel within rounding of it counts
+// must be decided exactly as the reference decides it -- sqrtf of the uncontracted
+// ((dx^2 + dy^2) + dz^2) against radius * radius_scale * final multiple
+// (src/grid_maker.cu:881-919) --, not on squares.  `cut` is that product.
+__device__ __forceinline__ float grad_scale_cut(const GradConsts& c, float dx, float dy, float dz,
+                                                float cut, float gridval) {
+  const float d2 = sq_distance_exact(dx, dy, dz);
+  const float e = __builtin_amdgcn_exp2f(d2 * c.exp_k);
+  return (sqrtf(d2) > cut) ? 0.f : c.gauss * e * gridval;
+}
+
+// Whether the kernels must take that path for this grid maker.
+inline bool cut_without_tail(const GridArg& g) { return g.frm <= g.grm; }
+
+// (CUT: the density jumps at its cut-off as well and takes the reference's predicates there)
+template <bool BINARY, bool CUT>
 __device__ __forceinline__ float point_density(const GridArg& g, float dx, float dy, float dz,
-                                               float ar2, float inv_ar2, float frm2, float grm2) {
-  return density<BINARY, false>(g, dx, dy, dz, BINARY ? ar2 : inv_ar2, 0.f, frm2, grm2);
+                                               float ar, float ar2, float inv_ar2, float frm2,
+                                               float grm2) {
+  return density<BINARY, CUT>(g, dx, dy, dz, BINARY ? ar2 : inv_ar2, ar, frm2, grm2);
 }
 
 constexpr int kRawBufferFlags = 0x00020000;   // untyped 32-bit elements, no swizzle (gfx9 family)
@@ -77,7 +94,7 @@ __device__ __forceinline__ float mul_zero_wins(float a, float b) { return mul_le
 // UNROTATE: the gradient is stored after Transform::backward(..., dotranslate = false) with the
 // example's quaternion and rotation centre, with the arithmetic of that call (transform.hip), so
 // that the result is the one the two calls give, bit for bit, with one launch less.
-template <bool UNROTATE>
+template <bool UNROTATE, bool CUT>
 __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_index, const float* __restrict__ radii,
@@ -143,9 +160,20 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
       const float core2 = g.grm * g.grm * ar * ar;
       const float reach2 = densityrad * densityrad;
       int lo0, lo1, lo2, ni, nj, nk;
-      reach_range(ox, ax, densityrad, inv_res, dim, lo0, ni);
-      reach_range(oy, ay, densityrad, inv_res, dim, lo1, nj);
-      reach_range(oz, az, densityrad, inv_res, dim, lo2, nk);
+      if (CUT) {
+        // the reference's index box: a voxel exactly at +reach on an axis is outside it
+        int hi0, hi1, hi2;
+        bounds_1d(ox, ax, densityrad, g.resolution, dim, lo0, hi0);
+        bounds_1d(oy, ay, densityrad, g.resolution, dim, lo1, hi1);
+        bounds_1d(oz, az, densityrad, g.resolution, dim, lo2, hi2);
+        ni = hi0 - lo0;
+        nj = hi1 - lo1;
+        nk = hi2 - lo2;
+      } else {
+        reach_range(ox, ax, densityrad, inv_res, dim, lo0, ni);
+        reach_range(oy, ay, densityrad, inv_res, dim, lo1, nj);
+        reach_range(oz, az, densityrad, inv_res, dim, lo2, nk);
+      }
       if (ni > 0 && nj > 0 && nk > 0 && ar > 0.f) {
         const float* chan = diff_b + (size_t)(int)tf * chan_stride;
         const int ncols = nj * nk;
@@ -192,7 +220,12 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
                   const float tail =
                       fmaxf(fmaf(quad_b, __builtin_amdgcn_rsqf(dist2), quad_a), 0.f);
                   float s = tail;
-                  if (!((tail_planes >> (i + u)) & 1ull)) {
+                  if (CUT) {
+                    // a Gaussian cut off without a tail: in or out by the reference's own test
+                    // (grad_scale_cut), nothing beyond
+                    const float d2 = sq_distance_exact(dx, dy, dz);
+                    s = (!live || sqrtf(d2) > densityrad) ? 0.f : __builtin_amdgcn_exp2f(d2 * exp_k);
+                  } else if (!((tail_planes >> (i + u)) & 1ull)) {
                     const float core = __builtin_amdgcn_exp2f(dist2 * exp_k);
                     s = dist2 <= core2 ? core : tail;
                   }
@@ -214,7 +247,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
             const int j = (int)(((float)cand + 0.5f) * inv_nk), k = cand - j * nk;
             const float dy = grid_coord(oy, lo1 + j, g.resolution) - ay;
             const float dz = grid_coord(oz, lo2 + k, g.resolution) - az;
-            const bool within = cand < ncols && dy * dy + dz * dz <= reach2;
+            const bool within = cand < ncols && dy * dy + dz * dz <= (CUT ? reach2 * 1.00001f : reach2);
             const unsigned long long m = __ballot(within);
             if (within) cols[pending + __popcll(m & ((1ull << lane) - 1ull))] = (j << 16) | k;
             pending += __popcll(m);
@@ -250,7 +283,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_index_kernel(
 
 // Vector types.  TG channels are handled per pass so that the per-lane type
 // gradient partials stay in registers.
-template <bool BINARY, bool RTI, int TG>
+template <bool BINARY, bool RTI, int TG, bool CUT>
 __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
     GridArg g, BatchArg batch, Vec3Arg centers, const float* __restrict__ coords,
     const float* __restrict__ type_vector, const float* __restrict__ radii,
@@ -291,9 +324,9 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
       const GradConsts gc = grad_consts(g, ar);
       const float inv_ar2 = gc.inv_ar2;
       const bool any = ar > 0.f && densityrad > 0.f;             // no extent: no gradient
-      // density and gradient scale vanish beyond the final radius; a binary sphere wider than
-      // its index box is cut by the box
-      const bool index_box = BINARY && g.frm < 1.0f;
+      // density and gradient scale vanish beyond the final radius; where the box decides which
+      // voxels count, the sweep follows the box
+      const bool index_box = needs_index_box(g, BINARY);
       for (int cbase = 0; cbase < T; cbase += TG) {
         const int nchan = min(TG, T - cbase);
         float tg[TG];
@@ -304,7 +337,7 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
           sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad, index_box,
                     [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
                         unsigned lane_off, bool live) {
-                      float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+                      float val = point_density<BINARY, CUT>(g, dx, dy, dz, ar, ar2, inv_ar2, frm2, grm2);
                       if (!live) val = 0.f;
                       const float* p = group + plane_off;
                       float weighted = 0.f;  // sum_t weight_t * diff_t at this voxel
@@ -316,7 +349,8 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
                           weighted = fmaf(tv[cbase + t], gv, weighted);
                         }
                       }
-                      const float sc = grad_scale(gc, dist2, weighted);
+                      const float sc = CUT ? grad_scale_cut(gc, dx, dy, dz, densityrad, live ? weighted : 0.f)
+                                           : grad_scale(gc, dist2, weighted);
                       gx = fmaf(dx, sc, gx);
                       gy = fmaf(dy, sc, gy);
                       gz = fmaf(dz, sc, gz);
@@ -348,14 +382,15 @@ __global__ __launch_bounds__(kBwdThreads) void backward_vector_kernel(
         if (ar > 0.f && densityrad > 0.f) {
           const float* chan = diff_b + (size_t)t * chan_stride;
           sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
-                      BINARY && g.frm < 1.0f,
+                      needs_index_box(g, BINARY),
                         [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
                             unsigned lane_off, bool live) {
                           const float gv = (chan + plane_off)[lane_off];
-                          float val = point_density<BINARY>(g, dx, dy, dz, ar2, inv_ar2, frm2, grm2);
+                          float val = point_density<BINARY, CUT>(g, dx, dy, dz, ar, ar2, inv_ar2, frm2, grm2);
                           if (!live) val = 0.f;
                           tgt = fmaf(val, gv, tgt);
-                          const float sc = grad_scale(gc, dist2, gv);
+                          const float sc = CUT ? grad_scale_cut(gc, dx, dy, dz, densityrad, live ? gv : 0.f)
+                                               : grad_scale(gc, dist2, gv);
                           tx = fmaf(dx, sc, tx);
                           ty = fmaf(dy, sc, ty);
                           tz = fmaf(dz, sc, tz);
@@ -394,14 +429,18 @@ hipError_t launch_vec(const GridArg& g, const BatchArg& batch, int nbatch, int l
                       const float* radii, const float* diff, float* atom_gradients,
                       float* type_gradients, hipStream_t stream) {
   dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
-  if (g.ntypes <= 8)
-    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 8>), grid, block, 0, stream, g, batch,
+  if (cut_without_tail(g))      // (a rare mode: one channel-group size serves it)
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 8, true>), grid, block, 0, stream, g,
+                       batch, centers, coords, type_vector, radii, diff, atom_gradients,
+                       type_gradients);
+  else if (g.ntypes <= 8)
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 8, false>), grid, block, 0, stream, g, batch,
                        centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
   else if (g.ntypes <= 16)
-    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 16>), grid, block, 0, stream, g, batch,
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 16, false>), grid, block, 0, stream, g, batch,
                        centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
   else
-    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 32>), grid, block, 0, stream, g, batch,
+    hipLaunchKernelGGL((backward_vector_kernel<BINARY, RTI, 32, false>), grid, block, 0, stream, g, batch,
                        centers, coords, type_vector, radii, diff, atom_gradients, type_gradients);
   return hipGetLastError();
 }
@@ -415,8 +454,12 @@ hipError_t launch_backward_index(const GridArg& g, const BatchArg& batch, int nb
   dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
   const Vec4Arg no_quats{nullptr, {1.f, 0.f, 0.f, 0.f}};
   const Vec3Arg no_centers{nullptr, {0.f, 0.f, 0.f}};
-  hipLaunchKernelGGL(backward_index_kernel<false>, grid, block, 0, stream, g, batch, centers,
-                     coords, type_index, radii, diff, atom_gradients, no_quats, no_centers);
+  if (cut_without_tail(g))
+    hipLaunchKernelGGL((backward_index_kernel<false, true>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, diff, atom_gradients, no_quats, no_centers);
+  else
+    hipLaunchKernelGGL((backward_index_kernel<false, false>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, diff, atom_gradients, no_quats, no_centers);
   return hipGetLastError();
 }
 
@@ -427,8 +470,12 @@ hipError_t launch_backward_index_unrotated(const GridArg& g, const BatchArg& bat
                                            const Vec4Arg& quats, const Vec3Arg& rot_centers,
                                            float* atom_gradients, hipStream_t stream) {
   dim3 grid(backward_blocks(launch_atoms), nbatch), block(kBwdThreads);
-  hipLaunchKernelGGL(backward_index_kernel<true>, grid, block, 0, stream, g, batch, centers,
-                     coords, type_index, radii, diff, atom_gradients, quats, rot_centers);
+  if (cut_without_tail(g))
+    hipLaunchKernelGGL((backward_index_kernel<true, true>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, diff, atom_gradients, quats, rot_centers);
+  else
+    hipLaunchKernelGGL((backward_index_kernel<true, false>), grid, block, 0, stream, g, batch, centers,
+                       coords, type_index, radii, diff, atom_gradients, quats, rot_centers);
   return hipGetLastError();
 }
 

@@ -60,10 +60,12 @@ GridArg grid_arg(const mg_gridmaker* g, int ntypes) {
 // per-atom index box.  That is indistinguishable from the reference when the
 // density reaches zero at the cut-off and the box is wider than the support.
 // A truncated Gaussian (negative gaussian_radius_multiple at construction:
-// no quadratic tail, final == gaussian multiple) or a binary sphere wider than
-// the box need the reference's exact predicates.
+// no quadratic tail, final == gaussian multiple) or a binary sphere that is not
+// narrower than the box (final multiple <= 1; at exactly 1 box and sphere
+// coincide and the rounding of the box's edges decides about voxels on them)
+// need the reference's exact predicates and its index box.
 bool needs_exact(const mg_gridmaker* g) {
-  if (g->binary) return g->final_radius_multiple < 1.0f;
+  if (g->binary) return g->final_radius_multiple <= 1.0f;
   return g->final_radius_multiple <= g->gaussian_radius_multiple;
 }
 

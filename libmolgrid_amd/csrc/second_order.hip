@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void relevance_kernel(
         const float* dens = density_grid + example + (size_t)(int)tf * chan_stride;
         const float* dif = diff + example + (size_t)(int)tf * chan_stride;
         sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
-                    BINARY && g.frm < 1.0f,
+                    needs_index_box(g, BINARY),
                     [&](float dx, float dy, float dz, float, unsigned plane_off, unsigned lane_off,
                         bool live) {
                       const float val = calc_point_reference<BINARY>(g, dx, dy, dz, ar);
@@ -153,10 +153,16 @@ __global__ __launch_bounds__(kThreads) void grad_grad_kernel(
       const float rcut = ar * g.frm, rcore = ar * g.grm;
       const float* dif = diff + example + (size_t)t * chan_stride;
       float* dd = diffdiff + example + (size_t)t * chan_stride;
-      sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
+      // (over the reference's index box: the second derivatives do not vanish at the cut-off, and
+      // the box leaves out a voxel that sits exactly at +reach on an axis)
+      sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad, true,
                 [&](float dx, float dy, float dz, float dist2, unsigned plane_off,
                     unsigned lane_off, bool live) {
-                  const float dist = sqrtf(dist2);
+                  // (the reference's own distance, src/grid_maker.cu:898-919: sqrtf of the
+                  // uncontracted sum of squares; the terms jump at both radii, so a voxel within
+                  // rounding of one must fall on the reference's side)
+                  const float rsq = sq_distance_exact(dx, dy, dz);
+                  const float dist = sqrtf(rsq);
                   if (!live || dist > rcut) return;   // density_grad_dist is NaN out here
                   const float G = (dif + plane_off)[lane_off];
                   // slope of the density along dist, the density, and with p = voxel - atom:

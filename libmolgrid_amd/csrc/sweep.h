@@ -197,9 +197,18 @@ __device__ __forceinline__ void sweep_reach(const GridArg& g, int lane, volatile
   }
 }
 
-// sweep_reach, or -- `index_box` -- the reference's index box for the radius `reach` (sweep_box): for
-// the one case in which that box is SMALLER than the support of the density, a binary sphere with
-// a final radius multiple below one, where the box decides which voxels count.
+// Whether the sweeps must follow the reference's index box (src/grid_maker.cu:66-79) instead of the
+// reach: the box is what decides which voxels count where it is NOT wider than the support of the
+// density or where the density does not fade to zero at its edge.  That is a binary sphere with a
+// final radius multiple of at most one (the box is smaller than the sphere, or coincides with it,
+// and then the rounding of its edges decides about the voxels on them), and a Gaussian cut off
+// without a tail (final multiple = Gaussian multiple): the box [floor(lo), ceil(hi)) leaves out a
+// voxel that sits exactly at +reach on an axis, where such a density and its gradient are not zero.
+__device__ __forceinline__ bool needs_index_box(const GridArg& g, bool binary) {
+  return (binary && g.frm <= 1.0f) || g.frm <= g.grm;
+}
+
+// sweep_reach, or -- `index_box` -- the reference's index box for the radius `reach` (sweep_box).
 template <typename Body>
 __device__ __forceinline__ void sweep_reach(const GridArg& g, int lane, volatile int* cols,
                                             float ox, float oy, float oz, float ax, float ay,

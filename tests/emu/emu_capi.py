@@ -40,6 +40,14 @@ def array(shape, dtype=np.float32, fill=None, tight=True):
     return a
 
 
+def release_all():
+    """Gives back every array handed out so far (their numpy views must not be used afterwards):
+    for runs of many cases in one process."""
+    for buf in _keep:
+        lib.emu_free(ctypes.addressof(buf))
+    del _keep[:]
+
+
 def put(x, dtype=np.float32):
     """Copy of x in guarded memory."""
     x = np.ascontiguousarray(x, dtype=dtype)

@@ -45,6 +45,17 @@ def test_hostile_inputs_return(emulated_library):
     assert "12 rounds returned" in p.stdout
 
 
+def test_randomised_parity(emulated_library):
+    """tests/emu/random_parity.py: the configuration itself is drawn -- grid size, resolution,
+    channel count, radius scale, radius multiples (truncated modes too), atoms on voxel centres
+    with radii that put voxels ON the cut-off -- and every kernel compared with the oracle under
+    the GPU tests' bounds (a few rounds here; thousands by hand, which is how the handling of a
+    Gaussian cut off without a tail and of a binary sphere as wide as its index box was found)."""
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_parity.py"), "40", "5"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+    assert p.returncode == 0 and "40 rounds passed" in p.stdout, p.stdout[-3000:]
+
+
 @pytest.mark.parametrize("checks", ["undefined", "address"])
 def test_run_time_checks(emulated_library, checks):
     """The same sources built again with clang's run-time checks, every report fatal, running the

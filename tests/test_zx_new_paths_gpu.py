@@ -130,3 +130,74 @@ def test_atom_lists_give_the_same_grids(mg, binary):
     out = torch.full(shape, 7.0, device="cuda")
     gm.forward_batch(v["offsets"], cen, c, t, r, out)
     assert torch.equal(out, plain)
+
+
+def _atoms_on_voxel_centres(res, dim, radius):
+    """Atoms on voxel centres of a grid centred at the origin: in the middle, at a face, at a corner."""
+    half = (dim - 1) * res / 2
+    idx = np.array([[dim // 2, dim // 2, dim // 2], [dim // 2, dim - 1, dim // 2 - 1], [0, 0, dim - 1],
+                    [dim // 2 - 3, dim // 2 + 2, 3]], np.float32)
+    coords = (idx * res - half).astype(np.float32)
+    return coords, np.full(len(coords), radius, np.float32)
+
+
+def test_truncated_gaussian_with_voxels_on_the_cut_off(mg):
+    """A Gaussian cut off without a tail (negative radius multiple) jumps at its cut-off.  With atoms
+    on voxel centres and a cut-off of exactly five voxels there are 30 voxels ON it per atom: the
+    reference counts those that its index box holds (the one at +5 voxels on an axis is outside,
+    src/grid_maker.cu:66-79) by sqrtf(dist^2) > cut.  Forward, backward (index and vector types) and
+    relevance must agree with the oracle there, which squares and a symmetric range do not."""
+    res, dim, T = 0.5, 32, 3
+    gm_args = (res, (dim - 1) * res, False, False, 1.0, -1.0)
+    coords, radii = _atoms_on_voxel_centres(res, dim, 2.5)
+    types = np.array([0, 1, 2, 1], np.float32)
+    og = oracle.GridMaker(*gm_args)
+    ref = og.forward((0, 0, 0), coords, types, radii, T)
+    got = gpu_forward(mg, gm_args, (0, 0, 0), coords, types, radii, T)
+    assert_close(got, ref, what="truncated Gaussian, forward")
+    rng = np.random.default_rng(3)
+    diff = rng.standard_normal(ref.shape).astype(np.float32)
+    gm = mg.GridMaker(*gm_args)
+    grads = torch.empty((len(coords), 3), device="cuda")
+    gm.backward((0, 0, 0), dev(coords), dev(types), dev(radii), dev(diff), grads)
+    ref32 = og.backward((0, 0, 0), coords, types, radii, diff)
+    ref64 = og.backward((0, 0, 0), coords, types, radii, diff, f64=True)
+    from test_backward_gpu import check_grads, noise_bound
+    check_grads(grads.cpu().numpy(), ref32, ref64,
+                noise_bound(og, (0, 0, 0), coords, types, radii, diff) + 1.0, "truncated Gaussian, backward")
+    # vector types: the same atoms with two-channel weights
+    tv = rng.uniform(0.2, 1.0, (len(coords), T)).astype(np.float32)
+    vgot = torch.empty(gm.grid_dimensions(T), device="cuda")
+    gm.forward((0, 0, 0), dev(coords), dev(tv), dev(radii), vgot)
+    assert_close(vgot.cpu().numpy(), og.forward((0, 0, 0), coords, tv, radii), what="truncated, vector forward")
+    ag, tg = torch.empty((len(coords), 3), device="cuda"), torch.empty((len(coords), T), device="cuda")
+    gm.backward((0, 0, 0), dev(coords), dev(tv), dev(radii), dev(diff), ag, tg)
+    ra, rt = og.backward((0, 0, 0), coords, tv, radii, diff, f64=True)
+    assert np.allclose(ag.cpu().numpy(), ra, rtol=1e-4, atol=1e-4), np.abs(ag.cpu().numpy() - ra).max()
+    assert np.allclose(tg.cpu().numpy(), rt, rtol=1e-4, atol=1e-4), np.abs(tg.cpu().numpy() - rt).max()
+    rel = torch.empty(len(coords), device="cuda")
+    gm.backward_relevance((0, 0, 0), dev(coords), dev(types), dev(radii), dev(ref), dev(diff), rel)
+    rref = og.backward_relevance((0, 0, 0), coords, types, radii, ref, diff)
+    assert np.allclose(rel.cpu().numpy(), rref, rtol=1e-4, atol=1e-4), np.abs(rel.cpu().numpy() - rref).max()
+
+
+@pytest.mark.parametrize("scale", [1.0, 1.3])
+def test_binary_sphere_that_coincides_with_its_index_box(mg, scale):
+    """Binary density with a final radius multiple of exactly one: the reference's index box has
+    the sphere's own radius, and voxels within rounding of the surface are decided by the rounding
+    of the box's edges.  Atoms on voxel centres with radii that put voxels on the surface, to the
+    last bit and one bit either side; bit-exact against the oracle, index and vector types."""
+    res, dim, T = 0.5, 24, 2
+    gm_args = (res, (dim - 1) * res, True, False, scale, -1.0)
+    coords, _ = _atoms_on_voxel_centres(res, dim, 1.0)
+    base = np.float32(2.5 / scale)
+    radii = np.array([base, np.nextafter(base, np.float32(9)), np.nextafter(base, np.float32(0)), base], np.float32)
+    types = np.array([0, 1, 0, 1], np.float32)
+    og = oracle.GridMaker(*gm_args)
+    got = gpu_forward(mg, gm_args, (0, 0, 0), coords, types, radii, T)
+    assert np.array_equal(got, og.forward((0, 0, 0), coords, types, radii, T))
+    tv = np.array([[1, 0.5], [0.25, 1], [1, 1], [0, 2]], np.float32)
+    gm = mg.GridMaker(*gm_args)
+    vgot = torch.empty(gm.grid_dimensions(T), device="cuda")
+    gm.forward((0, 0, 0), dev(coords), dev(tv), dev(radii), vgot)
+    assert np.array_equal(vgot.cpu().numpy(), og.forward((0, 0, 0), coords, tv, radii))
