@@ -213,7 +213,8 @@ int mg_forward_vector(const mg_gridmaker* g, int nbatch, const int32_t* atom_off
  * example (the reference's kernel scans them all per block,
  * src/grid_maker.cu:348-441).  The grids are the same bit for bit; the size is 0
  * for the configurations that do not use lists (type-indexed radii, truncated
- * densities).  `atoms_per_example` must be at least the largest example. */
+ * densities, more than 65,536 atoms per example).  `atoms_per_example` must be
+ * at least the largest example. */
 int mg_forward_vector_ws(const mg_gridmaker* g, int nbatch, const int32_t* atom_offsets,
                          int atoms_per_example, const float* grid_centers,
                          const float grid_center_host[3], const float* coords,

@@ -416,7 +416,7 @@ size_t mg_forward_vector_workspace_size(const mg_gridmaker* g, int nbatch, int a
                                         int ntypes) {
   if (g == nullptr || nbatch <= 0 || ntypes <= 0 || atoms_per_example <= 0) return 0;
   // only the matrix-core kernel (per-atom radii, density reaching zero at the cut-off) uses lists
-  if (g->radii_type_indexed || needs_exact(g)) return 0;
+  if (g->radii_type_indexed || needs_exact(g) || atoms_per_example > 65536) return 0;
   return forward_vector_workspace_bytes(nbatch, atoms_per_example, (int)g->dim);
 }
 

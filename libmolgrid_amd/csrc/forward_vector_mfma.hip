@@ -135,19 +135,22 @@ splat_vector_mfma_kernel(
   int segstart[kColWaves + 1];
   int ncand = 0;
 
-  // ---- scan: atoms [s0, s1) against the group's box -> per-wave index segments --------------
-  // With lists (a launch before this one has left, for every example and slab of four x planes,
-  // the atoms that can reach the slab's planes, in atom order), a workgroup scans its slab's list
-  // -- about a fifth of the example -- instead of all atoms.
+  // ---- scan: units [u0, u1) against the group's box -> per-wave index segments -----------------
+  // A unit is an atom of the example (its index), or -- with lists: a launch before this one has
+  // left, for every example and slab of four x planes, the atoms that can reach the slab's planes,
+  // in atom order -- a position of this slab's list, about a fifth of the example.  A segment
+  // entry is the atom's index relative to `base`, in 16 bits: the first atom of the window for
+  // windows of atoms, the first atom of the example for lists (which the launcher therefore
+  // builds for examples of up to 65,536 atoms only).  A window of kSuper units gives a wave at
+  // most kSeg of them, so its segment cannot overflow.
   const unsigned* const my_list =
       slab_lists != nullptr ? slab_lists + ((size_t)b * cols_per_side + x0 / kColXY) * list_stride : nullptr;
   const int my_listed = slab_lists != nullptr ? slab_counts[b * cols_per_side + x0 / kColXY] : 0;
-  auto scan = [&](int s0, int s1) -> bool {
-    // what is scanned: positions [0, total) of the list, or the atoms s0 + [0, total)
-    const int total = my_list != nullptr ? my_listed : s1 - s0;
-    const int quarter = (total + kColWaves - 1) / kColWaves;
+  const int unit_begin = my_list != nullptr ? 0 : begin, unit_end = my_list != nullptr ? my_listed : end;
+  auto scan = [&](int u0, int u1, int base) -> bool {
+    const int quarter = (u1 - u0 + kColWaves - 1) / kColWaves;
     int wcnt = 0;
-    const int wb = wave * quarter, we = min(total, wb + quarter);
+    const int wb = u0 + wave * quarter, we = min(u1, wb + quarter);
     constexpr int U = 2;
     for (int i0 = wb; i0 < we; i0 += kWave * U) {
       float rr[U], cx[U], cy[U], cz[U];
@@ -155,7 +158,7 @@ splat_vector_mfma_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int i = min(i0 + u * kWave + lane, we - 1);
-        at[u] = my_list != nullptr ? begin + (int)my_list[i] : s0 + i;
+        at[u] = my_list != nullptr ? begin + (int)my_list[i] : i;
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -169,12 +172,12 @@ splat_vector_mfma_kernel(
       for (int u = 0; u < U; ++u) {
         const int a = at[u];
         const float reach = rr[u] * g.radius_scale * (BINARY ? 1.0f : g.frm);
-        const bool p = (i0 + u * kWave + lane < we) && a >= s0 && a < s1 &&
+        const bool p = (i0 + u * kWave + lane < we) &&
                        box_distance2(cx[u], cy[u], cz[u], clx, gly, clz, chx, ghy, chz) <=
                            reach * reach * kCullSlack;
         const unsigned long long m = __ballot(p);
         const int pos = wcnt + __popcll(m & ((1ull << lane) - 1ull));
-        if (p && pos < kSeg) s_idx[wave][pos] = (unsigned short)(a - s0);
+        if (p && pos < kSeg) s_idx[wave][pos] = (unsigned short)(a - base);
         wcnt += __popcll(m);
       }
     }
@@ -251,8 +254,8 @@ splat_vector_mfma_kernel(
   }
   // whole example in one scan when its survivors fit; else passes of kSuper atoms per column
   bool one_pass = false;
-  if (end - begin <= 65536) one_pass = scan(begin, end);
-  const int pass_len = one_pass ? max(end - begin, 1) : kSuper;
+  if (end - begin <= 65536) one_pass = scan(unit_begin, unit_end, begin);
+  const int pass_len = one_pass ? max(unit_end - unit_begin, 1) : kSuper;
 
   // fixed positions of this thread in the staged write-out (float4 granules)
   constexpr int kItems = kStageCh * 16 * (kSlabZ / 4);               // 768 per round
@@ -277,8 +280,9 @@ splat_vector_mfma_kernel(
 #pragma unroll
           for (int h = 0; h < 2; ++h) sums[blk][t][h] = v4f{0.f, 0.f, 0.f, 0.f};
 
-      for (int s0 = begin; s0 < end; s0 += pass_len) {
-        if (!one_pass) scan(s0, min(end, s0 + kSuper));
+      for (int u0 = unit_begin; u0 < unit_end; u0 += pass_len) {
+        const int s0 = my_list != nullptr || one_pass ? begin : u0;   // what segment entries count from
+        if (!one_pass) scan(u0, min(unit_end, u0 + kSuper), s0);
         for (int c0 = 0; c0 < ncand; c0 += kRecChunk) {
           const int m = min(kRecChunk, ncand - c0);
           build_records(s0, c0, m, cbase, nchan);
@@ -533,7 +537,7 @@ hipError_t launch_forward_vector_mfma(const GridArg& g, const BatchArg& batch, i
   unsigned* lists = nullptr;
   int* counts = nullptr;
   const int list_stride = batch.per_example;
-  if (workspace != nullptr && list_stride > 0 &&
+  if (workspace != nullptr && list_stride > 0 && list_stride <= 65536 &&
       workspace_bytes >= forward_vector_workspace_bytes(nbatch, list_stride, g.dim)) {
     counts = static_cast<int*>(workspace);
     lists = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(workspace) +

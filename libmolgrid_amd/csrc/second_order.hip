@@ -85,8 +85,10 @@ __global__ __launch_bounds__(kThreads) void relevance_kernel(
       if (densityrad > 0.f) {
         const float* dens = density_grid + example + (size_t)(int)tf * chan_stride;
         const float* dif = diff + example + (size_t)(int)tf * chan_stride;
-        sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad,
-                    needs_index_box(g, BINARY),
+        // (over the reference's index box, always: the box leaves out a voxel that sits exactly
+        // at +reach on an axis, and although the atom's density is next to nothing there, so may
+        // be the grid's that it is divided by)
+        sweep_reach(g, lane, s_cols[wave], ox, oy, oz, ax, ay, az, densityrad, true,
                     [&](float dx, float dy, float dz, float, unsigned plane_off, unsigned lane_off,
                         bool live) {
                       const float val = calc_point_reference<BINARY>(g, dx, dy, dz, ar);

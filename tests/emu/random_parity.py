@@ -38,6 +38,13 @@ def draw(rng):
     grm = float(rng.choice([1.0, 1.0, 1.0, 0.7, 1.5, 2.0, -1.5, -0.5, -1.0]))
     scale = float(rng.choice([1.0, 1.0, 0.6, 1.3]))
     natoms = int(rng.choice([1, 2, 7, 30, 64, 65, 150]))
+    size = rng.random()
+    if size < 0.04:          # a grid of more than one z slab (64: slabs of 32 voxels), few atoms and channels
+        dim, ntypes, natoms = int(rng.choice([64, 65, 96])), min(ntypes, 2), min(natoms, 30)
+        dimension = (dim - 1) * res
+    elif size < 0.10:        # more atoms than the sort keeps in registers, than one chunk of records holds
+        dim, ntypes, natoms = min(dim, 24), min(ntypes, 5), int(rng.choice([700, 5000]))
+        dimension = (dim - 1) * res
     half = dimension / 2
     spread = half + float(rng.choice([0.0, 1.0, 3.0]))
     center = rng.uniform(-2, 2, 3).astype(np.float32) * float(rng.choice([0, 1, 10]))
@@ -201,6 +208,20 @@ def one_round(rng):
                                                                np.broadcast_to(m, got.shape)[i],
                                                                (coords[i[0]] - (center - dimension / 2)) / res,
                                                                vr if rti else vr[i[0]], tv[i[0]]))
+
+    # ---- second order (Gaussian densities only, src/grid_maker.cpp:559), few atoms: the oracle is slow
+    if not binary and n <= 65 and d["dim"] <= 33:
+        w = rng.standard_normal((n, 3)).astype(np.float32)
+        v = rng.standard_normal((n, T)).astype(np.float32)
+        dd, add, _ = ogv.backward_gradients(center, coords, tv, vr, vdiff, w, v)
+        sdd, sadd, _ = ogv.backward_gradients(center, coords, np.abs(tv), vr, np.abs(vdiff), np.abs(w), np.abs(v))
+        g_dd, g_add, g_tdd = E.array(vdiff.shape, fill=9.0), E.array((n, 3), fill=9.0), E.array((n, T), fill=9.0)
+        assert lib.mg_backward_gradients(ctypes.byref(gv), 1, None, n, None, E.f3(center), E.ptr(E.put(coords)),
+                                         E.ptr(E.put(tv)), E.ptr(E.put(vr)), T, E.ptr(E.put(vdiff)),
+                                         E.ptr(E.put(w)), E.ptr(E.put(v)), E.ptr(g_dd), E.ptr(g_add),
+                                         E.ptr(g_tdd), None) == 0
+        C.close_sums(g_dd, dd, np.abs(sdd) + 1.0, "diffdiff rti=%d " % rti + tag)
+        C.close_sums(g_add, add, np.abs(sadd) * 4 + 1.0, "atom_diffdiff rti=%d " % rti + tag)
 
     # ---- resampling of the density under a random rotation (small grids: the oracle is a loop) --
     if 2 <= d["dim"] <= 24 and T <= 8:

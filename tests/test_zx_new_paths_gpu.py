@@ -132,6 +132,37 @@ def test_atom_lists_give_the_same_grids(mg, binary):
     assert torch.equal(out, plain)
 
 
+@pytest.mark.parametrize("binary", [False, True])
+def test_atom_lists_longer_than_one_scan_window(mg, binary):
+    """9,000 atoms crowded into a grid of 8 voxels a side: every slab's list holds nearly all of
+    them, more than the splat kernel scans in one window and more than a wave's segment of
+    candidates holds, so the list is taken window by window (a quarter of a window per wave).  The
+    grids with lists equal those without, bit for bit, and the oracle's."""
+    from libmolgrid_amd import _capi
+    rng = np.random.default_rng(77)
+    n, T = 9000, 3
+    coords = rng.uniform(-4.5, 4.5, (n, 3)).astype(np.float32)
+    tv = (rng.uniform(0, 1.5, (n, T)) * (rng.random((n, T)) > 0.3)).astype(np.float32)
+    radii = rng.uniform(0.6, 2.2, n).astype(np.float32)
+    gm_args = (1.0, 7.0, binary)
+    gm = mg.GridMaker(*gm_args)
+    c, t, r = dev(coords), dev(tv), dev(radii)
+    shape = gm.grid_dimensions(T)
+    plain, listed = torch.full(shape, 5.0, device="cuda"), torch.full(shape, 6.0, device="cuda")
+    args = [gm._p, 1, None, n, None, _capi.f3((0.3, 0, -0.2)), c.data_ptr(), t.data_ptr(), r.data_ptr(), T]
+    assert _capi.lib.mg_forward_vector(*args, plain.data_ptr(), None) == 0
+    need = int(_capi.lib.mg_forward_vector_workspace_size(gm._p, 1, n, T))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    assert _capi.lib.mg_forward_vector_ws(*args, listed.data_ptr(), ws.data_ptr(), need, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(listed, plain)
+    ref = oracle.GridMaker(*gm_args).forward((0.3, 0, -0.2), coords, tv, radii)
+    if binary:
+        assert np.array_equal(listed.cpu().numpy(), ref)
+    else:
+        assert_close(listed.cpu().numpy(), ref, what="9,000 atoms in 8^3 voxels")
+
+
 def _atoms_on_voxel_centres(res, dim, radius):
     """Atoms on voxel centres of a grid centred at the origin: in the middle, at a face, at a corner."""
     half = (dim - 1) * res / 2
@@ -201,3 +232,34 @@ def test_binary_sphere_that_coincides_with_its_index_box(mg, scale):
     vgot = torch.empty(gm.grid_dimensions(T), device="cuda")
     gm.forward((0, 0, 0), dev(coords), dev(tv), dev(radii), vgot)
     assert np.array_equal(vgot.cpu().numpy(), og.forward((0, 0, 0), coords, tv, radii))
+
+
+def test_relevance_with_voxels_at_the_end_of_the_tail(mg):
+    """Relevance divides an atom's density by the grid's.  With atoms on voxel centres, five voxels
+    apart, and a final radius of exactly five voxels, the voxel at +5 on an axis sits at the very
+    end of the quadratic tail, where the atom's density is next to nothing -- and so is the
+    grid's, so the quotient is not small.  The reference's index box leaves that voxel out
+    (src/grid_maker.cu:66-79); so must the kernel."""
+    res, dim, T, steps = 0.5, 24, 2, 5
+    gm_args = (res, (dim - 1) * res, False, False, 1.0, 0.7)
+    og = oracle.GridMaker(*gm_args)
+    half = (dim - 1) * res / 2
+    m = dim // 2
+    idx = np.array([[m, m, m], [m - steps, m, m], [m, m + steps, m], [3, 4, 5]], np.float32)
+    coords = (idx * res - half).astype(np.float32)
+    for nudge in (0, 1):
+        r = np.float32(steps * res / float(og.p.final_radius_multiple))
+        if nudge:
+            r = np.nextafter(r, np.float32(9))
+        radii = np.full(4, r, np.float32)
+        types = np.array([0, 0, 0, 1], np.float32)
+        dens = og.forward((0, 0, 0), coords, types, radii, T)
+        diff = np.random.default_rng(9).standard_normal(dens.shape).astype(np.float32)
+        gm = mg.GridMaker(*gm_args)
+        rel = torch.empty(len(coords), device="cuda")
+        gm.backward_relevance((0, 0, 0), dev(coords), dev(types), dev(radii), dev(dens), dev(diff), rel)
+        ref = og.backward_relevance((0, 0, 0), coords, types, radii, dens, diff)
+        scale = og.backward_relevance((0, 0, 0), coords, types, radii, dens, np.abs(diff))
+        eps = float(np.finfo(np.float32).eps)
+        assert (np.abs(rel.cpu().numpy() - ref) <= 1e-6 + 1e-5 * np.abs(ref) + 64 * eps * scale).all(), \
+            (nudge, rel.cpu().numpy(), ref)
