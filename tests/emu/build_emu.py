@@ -85,5 +85,22 @@ def build(force=False, verbose=False):
     return LIB_PATH
 
 
+def build_cpp_api_test():
+    """tests/cpp/test_api.cpp (the C++ classes of include/libmolgrid) compiled against the emulation
+    and linked with the emulated library: the C++ host layer on the CPU."""
+    lib = build()
+    out = os.path.join(HERE, "test_api_emu")
+    src = os.path.join(ROOT, "tests", "cpp", "test_api.cpp")
+    deps = [src, lib] + [os.path.join(ROOT, "include", "libmolgrid", f)
+                         for f in os.listdir(os.path.join(ROOT, "include", "libmolgrid"))]
+    if os.path.exists(out) and all(os.path.getmtime(d) <= os.path.getmtime(out) for d in deps):
+        return out
+    subprocess.check_call([_compiler(), "-std=c++17", "-O1", "-g", "-Wno-unknown-attributes",
+                           "-Wno-ignored-attributes", "-I" + HERE, "-I" + os.path.join(ROOT, "include"),
+                           src, "-o", out, "-L" + HERE, "-l" + os.path.basename(lib)[3:-3],
+                           "-Wl,-rpath,$ORIGIN"])
+    return out
+
+
 if __name__ == "__main__":
     print(build(force=True, verbose="-v" in sys.argv))

@@ -119,6 +119,19 @@ inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipMalloc(void** p, size_t n) { *p = emu::allocate(n); return *p ? hipSuccess : hipErrorOutOfMemory; }
 template <class T> inline hipError_t hipMalloc(T** p, size_t n) { return hipMalloc((void**)p, n); }
 inline hipError_t hipFree(void* p) { emu::release(p); return hipSuccess; }
+// (host code of the C++ classes: "device" memory is host memory here)
+enum hipMemcpyKind { hipMemcpyHostToHost, hipMemcpyHostToDevice, hipMemcpyDeviceToHost,
+                     hipMemcpyDeviceToDevice, hipMemcpyDefault };
+inline hipError_t hipMemcpy(void* dst, const void* src, size_t n, hipMemcpyKind) {
+  if (n) std::memmove(dst, src, n);
+  return hipSuccess;
+}
+inline hipError_t hipMemset(void* dst, int value, size_t n) {
+  if (n) std::memset(dst, value, n);
+  return hipSuccess;
+}
+inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
+inline hipError_t hipSetDevice(int d) { return d == 0 ? hipSuccess : hipErrorInvalidDevice; }
 inline hipError_t hipGetSymbolAddress(void** p, const void* symbol) { *p = const_cast<void*>(symbol); return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emulated HIP error"; }
 template <class F> inline hipError_t hipFuncSetAttribute(F, hipFuncAttribute, int) { return hipSuccess; }

@@ -45,6 +45,18 @@ def test_hostile_inputs_return(emulated_library):
     assert "12 rounds returned" in p.stdout
 
 
+def test_cpp_classes_on_the_emulated_library(emulated_library):
+    """tests/cpp/test_api.cpp -- GridMaker, GridInterpolater, Transform, Grid / ManagedGrid and
+    CoordinateSet of include/libmolgrid, used the way the reference's own unit tests use its
+    classes -- compiled against the emulation's stand-in for the HIP runtime and linked with the
+    emulated library: the whole C++ host layer, device paths included, on the CPU."""
+    sys.path.insert(0, os.path.join(HERE, "emu"))
+    import build_emu
+    p = subprocess.run([build_emu.build_cpp_api_test(), "gpu"], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert p.returncode == 0 and "0 failure(s)" in p.stdout, p.stdout[-3000:]
+
+
 def test_randomised_parity(emulated_library):
     """tests/emu/random_parity.py: the configuration itself is drawn -- grid size, resolution,
     channel count, radius scale, radius multiples (truncated modes too), atoms on voxel centres
