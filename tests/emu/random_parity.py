@@ -170,6 +170,43 @@ def one_round(rng):
                                per_example=max(int(np.diff(off).max()), 1), nbatch=B)
         C.close(gotb, refb, "ragged batch " + tag, exact=binary)
 
+    # ---- the same ragged batch through the transform, the backward pass and the launch that also
+    # takes the gradients back through the rotation (bit-identical to the two calls)
+    if n >= 7:
+        quats = synth.random_quaternions(rng, B)
+        rot_c = rng.uniform(-2, 2, (B, 3)).astype(np.float32)
+        trans = rng.uniform(-1, 1, (B, 3)).astype(np.float32)
+        off32 = E.put(off, np.int32)
+        width = max(int(np.diff(off).max()), 1)
+        moved = E.array((n, 3), fill=9.0)
+        assert lib.mg_transform_forward(B, E.ptr(off32), width, E.ptr(E.put(quats)), E.f4((1, 0, 0, 0)),
+                                        E.ptr(E.put(rot_c)), E.f3((0, 0, 0)), E.ptr(E.put(trans)),
+                                        E.f3((0, 0, 0)), 1, E.ptr(E.put(coords)), E.ptr(moved), None) == 0
+        ref_moved = oracle.transform_forward_batch(off, quats, rot_c, trans, coords)
+        C.close(moved, ref_moved, "transform batch " + tag, exact=True)
+        bdiff = rng.standard_normal(refb.shape).astype(np.float32)
+        bref = og.backward_batch(off, centers, ref_moved, types, radii, bdiff)
+        gb = E.gridmaker(*gm_args)
+        bgot, bun = E.array((n, 3), fill=9.0), E.array((n, 3), fill=9.0)
+        bargs = [ctypes.byref(gb), B, E.ptr(off32), width, E.ptr(E.put(centers)), E.f3((0, 0, 0)),
+                 E.ptr(E.put(ref_moved)), E.ptr(E.put(types)), E.ptr(E.put(radii)), T, E.ptr(E.put(bdiff))]
+        assert lib.mg_backward_index(*bargs, E.ptr(bgot), None) == 0
+        magb = np.concatenate([
+            np.abs(og.backward(centers[b], ref_moved[off[b]:off[b + 1]], types[off[b]:off[b + 1]],
+                               radii[off[b]:off[b + 1]], np.abs(bdiff[b]), f64=True)).max(axis=1, keepdims=True)
+            if off[b + 1] > off[b] else np.zeros((0, 1)) for b in range(B)]) + 1e-30
+        allow = np.concatenate([
+            tail_allowance(og, centers[b], ref_moved[off[b]:off[b + 1]],
+                           (lambda a, t, lo=off[b]: radii[lo + a]),
+                           onehot[off[b]:off[b + 1]], bdiff[b])[0] for b in range(B)])
+        err = np.abs(np.asarray(bgot, np.float64) - bref)
+        assert (err <= C.ATOL + C.RTOL * np.abs(bref) + 64 * EPS * magb + 4 * allow).all(), \
+            "backward batch %s: worst %g" % (tag, float(err.max()))
+        assert lib.mg_backward_index_unrotated(*bargs, E.ptr(E.put(quats)), E.f4((1, 0, 0, 0)), E.ptr(E.put(rot_c)),
+                                               E.f3((0, 0, 0)), E.ptr(bun), None) == 0
+        C.close(bun, oracle.transform_backward_batch(off, quats, rot_c, trans, np.array(bgot), dotranslate=False),
+                "fused un-rotation " + tag, exact=True)
+
     # ---- vector types: forward (atom lists or not), backward -----------------------------------
     rti = bool(rng.random() < 0.25)
     sparse = float(rng.choice([0.0, 0.5, 0.9]))

@@ -66,6 +66,11 @@ def test_randomised_parity(emulated_library):
     p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_parity.py"), "40", "5"],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
     assert p.returncode == 0 and "40 rounds passed" in p.stdout, p.stdout[-3000:]
+    # the same for resampling: grid sizes, resolution ratios, centres, shifts beyond the input,
+    # axis-aligned and random rotations (tests/emu/random_resample.py; 1,800 rounds by hand)
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_resample.py"), "40", "5"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+    assert p.returncode == 0 and "40 rounds passed" in p.stdout, p.stdout[-3000:]
 
 
 @pytest.mark.parametrize("checks", ["undefined", "address"])
