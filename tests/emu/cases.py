@@ -18,6 +18,7 @@ import synth  # noqa: E402
 
 lib = E.lib
 RTOL, ATOL = 1e-5, 1e-6
+STATIC_BYTES = 16 << 20      # MG_STATIC_SCRATCH_BYTES of include/molgrid_hip.h
 _checked = [0]
 
 

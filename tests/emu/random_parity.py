@@ -128,6 +128,13 @@ def one_round(rng):
     lib.mg_forward_index_paged(0)
     plain = np.array(C.forward_index(gm_args, center, coords, types, radii, T))
     C.close(plain, ref, "forward " + tag, exact=binary)
+    # the library's own workspace, or the entry point that allocates nothing (when the case fits
+    # its fixed scratch memory): the same grid bit for bit
+    variant = str(rng.choice(["cached", "static"]))
+    g0 = E.gridmaker(*gm_args)
+    if variant == "cached" or lib.mg_forward_index_workspace_size(ctypes.byref(g0), 1, n, T) <= C.STATIC_BYTES:
+        other = C.forward_index(gm_args, center, coords, types, radii, T, variant=variant)
+        C.close(other, plain, "forward, %s workspace, " % variant + tag, exact=True)
     lib.mg_forward_index_paged(1)
     paged = C.forward_index(gm_args, center, coords, types, radii, T)
     lib.mg_forward_index_paged(0)
