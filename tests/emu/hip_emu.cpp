@@ -334,6 +334,31 @@ bool buffer_ok(const Rsrc& r, uint32_t offset, uint32_t size, bool store) {
 }  // namespace emu
 
 // ---- what the tests call ---------------------------------------------------------------------------
+namespace emu {
+// see hip_emu.h: the exact result, or its neighbour one unit in the last place away
+float approx(float exact) {
+  static const int mode = [] {
+    const char* m = std::getenv("EMU_APPROX");
+    if (m == nullptr) return 0;
+    return !std::strcmp(m, "up") ? 1 : !std::strcmp(m, "down") ? 2 : !std::strcmp(m, "hash") ? 3 : 0;
+  }();
+  if (mode == 0 || exact == 0.0f || !std::isfinite(exact)) return exact;
+  int step = mode == 1 ? 1 : -1;
+  if (mode == 3) {
+    // like the hardware: the same result for the same value every time, off either way or not at all
+    uint32_t h;
+    std::memcpy(&h, &exact, 4);
+    h *= 0x9e3779b1u;
+    h ^= h >> 15;
+    h *= 0x85ebca77u;
+    h ^= h >> 13;
+    step = (int)(h % 3u) - 1;
+    if (step == 0) return exact;
+  }
+  return std::nextafter(exact, step > 0 ? INFINITY : -INFINITY);
+}
+}  // namespace emu
+
 extern "C" {
 void* emu_alloc(size_t bytes) { return emu::allocate(bytes, 256); }
 // the block ends within 15 bytes of an inaccessible page: an overrun faults

@@ -151,11 +151,19 @@ inline double __hiloint2double(int hi, int lo) {
 }
 inline int __popcll(unsigned long long v) { return __builtin_popcountll(v); }
 inline int __popc(unsigned v) { return __builtin_popcount(v); }
-inline float __expf(float x) { return expf(x); }
-#define __builtin_amdgcn_exp2f(x) exp2f(x)
-#define __builtin_amdgcn_sqrtf(x) sqrtf(x)
-#define __builtin_amdgcn_rsqf(x) (1.0f / sqrtf(x))
-#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+// The hardware's approximate instructions (v_exp_f32, v_sqrt_f32, v_rsq_f32, v_rcp_f32: about one
+// unit in the last place) are the exact results here, moved -- when the environment variable
+// EMU_APPROX is "up", "down" or "hash" -- by one unit in the last place up, down, or up, down or
+// not at all as a hash of the value decides (unbiased and repeatable, like the hardware; "up" and
+// "down" bias every term of a sum the same way, which no tolerance on long sums survives):
+// whatever a kernel builds on them (culls with a slack, index arithmetic through a
+// reciprocal, the bit-exact binary paths, which must not use them at all) has to hold then too.
+namespace emu { float approx(float exact); }
+inline float __expf(float x) { return emu::approx(expf(x)); }
+#define __builtin_amdgcn_exp2f(x) emu::approx(exp2f(x))
+#define __builtin_amdgcn_sqrtf(x) emu::approx(sqrtf(x))
+#define __builtin_amdgcn_rsqf(x) emu::approx(1.0f / sqrtf(x))
+#define __builtin_amdgcn_rcpf(x) emu::approx(1.0f / (x))
 #define __builtin_amdgcn_s_setprio(x) ((void)0)
 #define __builtin_amdgcn_s_sleep(x) ((void)0)
 
