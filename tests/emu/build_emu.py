@@ -17,6 +17,10 @@ SOURCES = ["capi.hip", "transform.hip", "convert.hip", "forward_sorted.hip", "fo
 # misaligned accesses), "list" the same but reporting and going on (to see every place at once),
 # "address" the address checks (every LDS array -- static storage here -- and every stack array gets
 # poisoned neighbours, so an access through a pointer that leaves its array is caught as well).
+# EMU_CONTRACT=1: a build that contracts a * b + c into one fused operation wherever the source
+# allows it, as the device compiler does by default (the plain build contracts nothing): the paths
+# that must match the reference bit for bit have to say so themselves (fp contract(off)).
+CONTRACT = os.environ.get("EMU_CONTRACT", "") not in ("", "0")
 SANITIZE = os.environ.get("EMU_SANITIZE", "")
 if SANITIZE in ("0",):
     SANITIZE = ""
@@ -27,6 +31,8 @@ else:
     SAN_FLAGS = ["-fsanitize=undefined,float-cast-overflow", "-fno-sanitize=vptr,function",
                  "-fsanitize-recover=all" if SANITIZE == "list" else "-fno-sanitize-recover=all"]
     TAG = "ubsan"
+if CONTRACT and not SANITIZE:
+    SANITIZE, TAG, SAN_FLAGS = "contract", "contract", []
 LIB_PATH = os.path.join(HERE, "libmolgrid_emu_%s.so" % TAG if SANITIZE else "libmolgrid_emu.so")
 
 
@@ -59,6 +65,8 @@ def build(force=False, verbose=False):
              "-I" + HERE, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
     if SANITIZE:
         flags += SAN_FLAGS
+    if CONTRACT:
+        flags = [f for f in flags if f != "-ffp-contract=off"] + ["-ffp-contract=fast-honor-pragmas", "-mfma"]
     procs = []
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
@@ -78,7 +86,7 @@ def build(force=False, verbose=False):
             print(out)
         objs.append(obj)
     link = []
-    if SANITIZE:      # the checks' runtime as a shared library, found beside the compiler
+    if SANITIZE and SAN_FLAGS:      # the checks' runtime as a shared library, found beside the compiler
         rt = subprocess.check_output([cxx, "-print-resource-dir"], text=True).strip() + "/lib/linux"
         link = SAN_FLAGS + ["-shared-libsan", "-Wl,-rpath," + rt]
     subprocess.check_call([cxx, "-shared", "-fPIC"] + link + objs + ["-o", LIB_PATH])

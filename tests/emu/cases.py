@@ -536,7 +536,10 @@ def group_interpolate():
         lib.mg_interpolate_force_gather(1)
         gathered = interpolate(in_res, in_a, out_res, out_a, grids, quats, shifts, centers)
         lib.mg_interpolate_force_gather(0)
-        close(gathered, got, "gather path equals staged path", exact=True)
+        # (bit for bit when both kernels round the lerps alike: in the plain build, where nothing is
+        # contracted, and on the device, whose compiler contracts them the same way in both -- the
+        # GPU test asserts it --; the host compiler of the contracting build does not)
+        close(gathered, got, "gather path equals staged path", exact=not os.environ.get("EMU_CONTRACT"))
 
 
 def group_config0():

