@@ -159,7 +159,28 @@ void describe_and_abort(const char* what) {
   _exit(86);
 }
 
+}  // namespace
+}  // namespace emu
+// bounds of the section that holds every __shared__ array (hip_emu.h), provided by the linker
+extern "C" char __start_emu_lds[] __attribute__((weak));
+extern "C" char __stop_emu_lds[] __attribute__((weak));
+namespace emu {
+namespace {
+
+// EMU_ORDER=reverse: threads (hence waves) and workgroups are run last to first.  Between two
+// meeting points a thread runs alone, so the results may not depend on who goes first: if they do,
+// a barrier is missing, or a workgroup relies on another.
+bool reverse_order() {
+  static const bool on = [] {
+    const char* m = std::getenv("EMU_ORDER");
+    return m != nullptr && !std::strcmp(m, "reverse");
+  }();
+  return on;
+}
+
 void run_block(int nthreads) {
+  if (__start_emu_lds != nullptr && __stop_emu_lds > __start_emu_lds)
+    std::memset(__start_emu_lds, 0xCB, (size_t)(__stop_emu_lds - __start_emu_lds));
   threads_total = threads_live = nthreads;
   barrier_arrived = 0;
   const int nwaves = (nthreads + 63) / 64;
@@ -174,8 +195,8 @@ void run_block(int nthreads) {
   uint64_t seen = progress;
   int idle_passes = 0;
   while (threads_live > 0) {
-    for (int t = 0; t < nthreads; ++t) {
-      Fiber& f = fibers[t];
+    for (int i = 0; i < nthreads; ++i) {
+      Fiber& f = fibers[reverse_order() ? nthreads - 1 - i : i];
       if (f.done) continue;
       if (f.wait_on != nullptr && *f.wait_on == f.wait_val) continue;
       running = &f;
@@ -228,9 +249,13 @@ void launch(dim3 grid, dim3 block, size_t shared_bytes, const std::function<void
   body_of_launch = &body;
   std::vector<char> shared(shared_bytes + 64);
   dynamic_shared = shared.data();
-  for (unsigned bz = 0; bz < grid.z; ++bz)
-    for (unsigned by = 0; by < grid.y; ++by)
-      for (unsigned bx = 0; bx < grid.x; ++bx) {
+  const bool backwards = reverse_order();
+  for (unsigned iz = 0; iz < grid.z; ++iz)
+    for (unsigned iy = 0; iy < grid.y; ++iy)
+      for (unsigned ix = 0; ix < grid.x; ++ix) {
+        const unsigned bx = backwards ? grid.x - 1 - ix : ix, by = backwards ? grid.y - 1 - iy : iy,
+                       bz = backwards ? grid.z - 1 - iz : iz;
+        std::memset(shared.data(), 0xCB, shared.size());     // dynamic LDS starts as garbage too
         for (size_t t = 0; t < nthreads; ++t) {
           Ctx& c = fibers[t].ctx;
           c.tid = make_uint3((unsigned)(t % block.x), (unsigned)((t / block.x) % block.y),

@@ -26,7 +26,10 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
-#define __shared__ static
+// (all LDS arrays go into one section of the library, which the emulator fills with 0xCB bytes
+// before every workgroup: a kernel that reads LDS it has not written sees garbage, as on the
+// hardware, not the zeros of static storage or the previous workgroup's leftovers)
+#define __shared__ static __attribute__((section("emu_lds")))
 #define __align__(n) __attribute__((aligned(n)))
 #define __constant__ static const
 #define amdgpu_waves_per_eu(...) unused

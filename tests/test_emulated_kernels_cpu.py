@@ -59,6 +59,21 @@ def test_one_unit_in_the_last_place_of_the_approximate_instructions(emulated_lib
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
 
 
+def test_threads_and_workgroups_run_last_to_first(emulated_library):
+    """Between two meeting points (a barrier, a cross-lane operation) an emulated thread runs alone,
+    and normally thread 0 goes first.  EMU_ORDER=reverse runs threads, hence waves, and workgroups
+    last to first: results that depend on who goes first -- a missing barrier, a workgroup that
+    relies on another -- change.  (In every mode the emulator fills all LDS with 0xCB before a
+    workgroup starts, so neither zeros nor the previous workgroup's leftovers can be relied on.)"""
+    env = dict(os.environ, EMU_ORDER="reverse")
+    for args in (["cases.py", "forward_paged"], ["cases.py", "forward_batch"], ["cases.py", "forward_vector"],
+                 ["cases.py", "backward_vector"], ["cases.py", "second_order"], ["cases.py", "interpolate"],
+                 ["random_parity.py", "15", "6"]):
+        p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
+        assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
+
+
 def test_with_fused_multiply_adds(emulated_library):
     """The device compiler turns a * b + c into one fused operation wherever the source lets it; the
     plain emulated build fuses nothing.  A second build (EMU_CONTRACT=1) fuses like the device
