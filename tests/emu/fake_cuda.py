@@ -156,7 +156,7 @@ def activate():
             return real_generator.__new__(cls)
 
     torch.Generator = HostGenerator
-    for name in ("empty", "zeros", "ones", "full", "randn", "rand", "arange", "tensor"):
+    for name in ("empty", "zeros", "ones", "full", "randn", "rand", "randint", "arange", "tensor", "linspace"):
         setattr(torch, name, _factory(getattr(torch, name)))
     real_as_tensor = torch.as_tensor
     torch.as_tensor = real_as_tensor
