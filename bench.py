@@ -469,9 +469,11 @@ def run_candidates(args):
 CANDIDATE_COMMAND = [sys.executable, os.path.abspath(__file__)]
 
 
-def candidates_from_child(args, timeout_s=900):
+def candidates_from_child(args, timeout_s=150):
     """Runs `bench.py --candidates` with this run's sizes and returns its JSON lines (those it
-    wrote before it ended, however it ended) and a note on how it ended."""
+    wrote before it ended, however it ended) and a note on how it ended.  The child gets two and a
+    half minutes (it needs about one, most of it the import of torch): a run that prints nothing
+    for longer than that looks hung from outside."""
     import subprocess
     cmd = CANDIDATE_COMMAND + ["--candidates", "--steps", str(args.steps), "--warmup", str(args.warmup),
                                "--batch", str(args.batch)]
@@ -480,6 +482,7 @@ def candidates_from_child(args, timeout_s=900):
         if on:
             cmd.append(flag)
     note = None
+    print("bench.py: timing the other step variants in a child process ...", file=sys.stderr, flush=True)
     try:
         p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
                            timeout=timeout_s)
