@@ -427,33 +427,14 @@ def run_candidates(args):
             emit({"candidate": name, "error": repr(e)[:200]})
 
     it = max(args.steps, 10)
-    for write_out in ("per_wave", "paged"):
-        prefix = ""
-        if write_out == "paged":
-            if args.no_autotune:
-                break
-            # the paged write-out: its grids bit for bit, the forward call's time with each, and
-            # the store skeleton of each (the same call with every atom ignored)
-            check = {}
-            try:
-                w.k_transform()
-                check["per_wave_ms"] = round(event_ms(w.k_forward, it), 4)
-                torch.cuda.synchronize()
-                per_wave_grid = grid.clone()
-                types_none = torch.full_like(w.types, -1.0)
-                check["per_wave_stores_ms"] = round(event_ms(lambda: w.k_forward_no_atoms(types_none), it), 4)
-                _capi.lib.mg_forward_index_paged(1)
-                check["paged_ms"] = round(event_ms(w.k_forward, it), 4)
-                torch.cuda.synchronize()
-                check["identical"] = bool(torch.equal(grid, per_wave_grid))
-                check["paged_stores_ms"] = round(event_ms(lambda: w.k_forward_no_atoms(types_none), it), 4)
-                del per_wave_grid, types_none
-            except Exception as e:
-                check["error"] = repr(e)[:200]
-            emit({"write_out_check": check})
-            if not check.get("identical"):
-                break
-            prefix = "paged/"
+    lib = _capi.lib
+
+    def select(instance):
+        lib.mg_forward_index_paged(1 if "paged" in instance else 0)
+        lib.mg_forward_index_core_skip(1 if "core" in instance else 0)
+
+    def step_variants(prefix, with_eager):
+        if with_eager:
             candidate(prefix + "serial_eager", w.step_serial, False)
         if not args.no_graph:
             candidate(prefix + "serial_graph", w.step_serial, True)
@@ -461,7 +442,48 @@ def run_candidates(args):
             candidate(prefix + "overlapped_eager", w.step_overlapped, False)
             if not args.no_graph:
                 candidate(prefix + "overlapped_graph", w.step_overlapped, True)
-    _capi.lib.mg_forward_index_paged(0)
+
+    # 1. the library's default instance of the splat launch, enqueued the other ways
+    select("per_wave")
+    step_variants("", False)
+    # 2. the other instances of the splat launch -- the paged write-out, tail-only blocks without
+    # the exponential, both --: their grids bit for bit, the forward call's time with each, and
+    # the store skeleton of either write-out (the same call with every atom ignored)
+    if not args.no_autotune:
+        check = {"identical": {}}
+        try:
+            w.k_transform()
+            check["per_wave_ms"] = round(event_ms(w.k_forward, it), 4)
+            torch.cuda.synchronize()
+            default_grid = grid.clone()
+            types_none = torch.full_like(w.types, -1.0)
+            check["per_wave_stores_ms"] = round(event_ms(lambda: w.k_forward_no_atoms(types_none), it), 4)
+            for instance in ("core", "paged", "paged_core"):
+                try:
+                    select(instance)
+                    grid.zero_()
+                    check[instance + "_ms"] = round(event_ms(w.k_forward, it), 4)
+                    torch.cuda.synchronize()
+                    check["identical"][instance] = bool(torch.equal(grid, default_grid))
+                    if instance == "paged":
+                        check["paged_stores_ms"] = round(event_ms(lambda: w.k_forward_no_atoms(types_none), it), 4)
+                except Exception as e:
+                    check[instance + "_error"] = repr(e)[:200]
+                    check["identical"][instance] = False
+            del default_grid, types_none
+        except Exception as e:
+            check["error"] = repr(e)[:200]
+        select("per_wave")
+        emit({"write_out_check": check})
+        # 3. the fastest of them that gives the same grids, enqueued every way
+        valid = [i for i in ("core", "paged", "paged_core")
+                 if check["identical"].get(i) and (i + "_ms") in check]
+        if valid and "per_wave_ms" in check:
+            fastest = min(valid, key=lambda i: check[i + "_ms"])
+            if check[fastest + "_ms"] < check["per_wave_ms"]:
+                select(fastest)
+                step_variants(fastest + "/", True)
+                select("per_wave")
     emit({"done": True})
 
 
@@ -712,25 +734,20 @@ def main():
     if child_note is not None:
         step_variants["candidates_note"] = child_note
     if write_out is not None:
-        write_out["used"] = "paged" if best.startswith("paged/") else "per_wave"
-        if write_out.get("identical") and "paged_ms" in write_out:
-            # the forward call with the paged write-out (bit-identical grids), same event timing,
-            # measured in the child; the figures above it in this object are the default's
-            pg = fwd_bytes / (write_out["paged_ms"] * 1e-3) / 1e9
-            paged = {"avg_launch_ms": write_out["paged_ms"], "achieved": round(pg, 1),
-                     "frac": round(pg / HBM_PEAK_GBS, 4),
-                     "forward_call_all_atoms_ignored_ms": write_out.get("paged_stores_ms")}
-            if best.startswith("paged/") and dominant_fwd:
-                # `value` is from a step with the paged write-out: the headline figures of this
-                # object are that call's, the default's move aside (the committed counter summary
-                # covers the default only, so no measured traffic for this one)
-                roofline["per_wave_write_out"] = {k: roofline[k] for k in
-                                                  ("avg_launch_ms", "achieved", "frac", "traffic")}
-                roofline.update(avg_launch_ms=paged["avg_launch_ms"], achieved=paged["achieved"],
-                                frac=paged["frac"], traffic=None)
-                roofline["write_out"] = "paged"
-            else:
-                roofline["paged_write_out"] = paged
+        used = best.split("/")[0] if "/" in best else "per_wave"
+        write_out["used"] = used
+        if used != "per_wave" and dominant_fwd and (used + "_ms") in write_out:
+            # `value` is from a step whose splat launch is another instance of the kernel (same grids
+            # bit for bit, timed in the child with the same events): the headline figures of this
+            # object are that call's, the default's move aside (the committed counter summary covers
+            # the default only, so no measured traffic for this one)
+            ms_used = write_out[used + "_ms"]
+            gbs = fwd_bytes / (ms_used * 1e-3) / 1e9
+            roofline["per_wave_write_out"] = {k: roofline[k] for k in
+                                              ("avg_launch_ms", "achieved", "frac", "traffic")}
+            roofline.update(avg_launch_ms=ms_used, achieved=round(gbs, 1),
+                            frac=round(gbs / HBM_PEAK_GBS, 4), traffic=None)
+            roofline["write_out"] = used
 
     out = {
         "metric": "grids/sec, 28x48^3 fp32 batch 50, fwd + atom-grad bwd; % of HBM roofline",
@@ -741,8 +758,8 @@ def main():
         "warmup": args.warmup,
         # which way of enqueueing the step `value` is from (step_variants lists all of them):
         # serial = the reference's order on one stream, overlapped = the sort launch beside the
-        # backward pass; eager = launch by launch, graph = one captured HIP graph; "paged/" = with
-        # the paged write-out of the splat launch
+        # backward pass; eager = launch by launch, graph = one captured HIP graph; a prefix such as
+        # "paged/" = with that instance of the splat launch (forward_write_out lists them)
         "launch": best,
         "ms_per_step": round(ms_per_step, 4),
         # wall time the host needs to enqueue a step (the timed loop before its synchronize): when

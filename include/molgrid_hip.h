@@ -194,6 +194,16 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
  * returns the previous setting. */
 int mg_forward_index_paged(int on);
 
+/* No counterpart in the reference.  1 = the splat launch of mg_forward_index*
+ * for a Gaussian density (fast predicates) takes the kernel instances whose cull
+ * also marks the blocks of four voxels that the Gaussian core of an atom can
+ * reach, and that skip the exponential in the other blocks of its reach (about
+ * half of them on the benchmark batch), 0 = every block evaluates both
+ * branches.  The grids are the same bit for bit.  Process-wide; returns the
+ * previous setting.  Off by default: the instances without it are the ones
+ * that have been timed. */
+int mg_forward_index_core_skip(int on);
+
 /* GridMaker::forward, vector types; replaces forward_gpu_vec and its launcher
  * (src/grid_maker.cu:348-441), values of src/grid_maker.cpp:214-271.
  *   type_vector [n, ntypes]; radii [n], or [nbatch, ntypes] when

@@ -20,6 +20,7 @@ EXPORTED_SYMBOLS = (
     "mg_version", "mg_error_string", "mg_trace_ranges", "mg_gridmaker_init", "mg_transform_forward",
     "mg_transform_backward", "mg_forward_index", "mg_forward_index_ws",
     "mg_forward_index_workspace_size", "mg_forward_index_static", "mg_forward_index_paged",
+    "mg_forward_index_core_skip",
     "mg_forward_index_sort", "mg_forward_index_splat", "mg_forward_vector_ws",
     "mg_forward_vector_workspace_size", "mg_forward_vector", "mg_backward_index",
     "mg_backward_index_unrotated",
@@ -98,6 +99,7 @@ def declare(lib):
     lib.mg_widen.argtypes = [_vp, _vp, ctypes.c_size_t, _vp]
     lib.mg_interpolate_force_gather.argtypes = [_i]
     lib.mg_forward_index_paged.argtypes = [_i]
+    lib.mg_forward_index_core_skip.argtypes = [_i]
     lib.mg_trace_ranges.argtypes = [_i]
     for name in EXPORTED_SYMBOLS:
         fn = getattr(lib, name)

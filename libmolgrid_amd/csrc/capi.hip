@@ -411,6 +411,7 @@ int mg_forward_index_static(const mg_gridmaker* g, int nbatch, const int32_t* at
 }
 
 int mg_forward_index_paged(int on) { return set_forward_paged(on); }
+int mg_forward_index_core_skip(int on) { return set_forward_core_skip(on); }
 
 size_t mg_forward_vector_workspace_size(const mg_gridmaker* g, int nbatch, int atoms_per_example,
                                         int ntypes) {

@@ -361,7 +361,10 @@ __device__ __forceinline__ int block_above(float bottom) {
   return (int)fminf(fmaxf(ceilf(bottom), 0.f), 32.f);
 }
 
-template <bool BINARY, bool EXACT, int COLS, bool PAGED>
+// CORE (Gaussian density, fast predicates only): the cull also finds, per column, the blocks that
+// the Gaussian core of an atom can reach; the blocks of its reach beyond them take the quadratic
+// tail without evaluating the exponential.  The same sums bit for bit.
+template <bool BINARY, bool EXACT, int COLS, bool PAGED, bool CORE = false>
 __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sorted_kernel(
     GridArg g, const float4* __restrict__ slot_info, const int* __restrict__ cand,
     const float4* __restrict__ records, int capacity, float* __restrict__ out,
@@ -618,7 +621,7 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
           // conversion out of range)
           const int qhi = block_below(top, last_block), qlo = block_above(bottom);
           if (qlo <= qhi) mask[col] = (2u << qhi) - (1u << qlo);
-          if (!BINARY && !EXACT) {
+          if (CORE) {
             // bits 16..27: the blocks that the Gaussian core of the atom (u <= grm^2) can reach,
             // a subset of the above; the others take the quadratic tail without the exponential
             const float cz2 = core2 - (ex * ex + ey * ey);
@@ -669,7 +672,7 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
 #pragma unroll
         for (int col = 0; col < COLS; ++col) {
           const unsigned both = (unsigned)__builtin_amdgcn_readlane((int)mask[col], src);
-          const unsigned reach = both & 0xffffu, core = both >> 16;
+          const unsigned reach = CORE ? both & 0xffffu : both, core = both >> 16;
           if (reach == 0) continue;
           touched |= 1u << col;
           const float dy = vy[col] - ry;
@@ -703,14 +706,21 @@ __global__ __launch_bounds__(PAGED ? kPagedWaves * kWave : kWave) void splat_sor
               } else {
                 const float u = fmaf(dz, dz, dxy2) * rw;
                 if (u <= frm2) {
-                  const float su = __builtin_amdgcn_sqrtf(u);
-                  float val = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
-                  if ((core >> q) & 1u) {          // scalar test: else no voxel of the block
-                    keep_branch();
-                    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);   // is in the core
-                    val = (u <= grm2) ? gauss : val;
+                  if (CORE) {
+                    const float su = __builtin_amdgcn_sqrtf(u);
+                    float val = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+                    if ((core >> q) & 1u) {        // scalar test: else no voxel of the block
+                      keep_branch();
+                      const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);   // is in the core
+                      val = (u <= grm2) ? gauss : val;
+                    }
+                    acc[col][q] += val;
+                  } else {
+                    const float gauss = __builtin_amdgcn_exp2f(u * kNeg2Log2e);
+                    const float su = __builtin_amdgcn_sqrtf(u);
+                    const float quad = fmaxf(fmaf(g.A, u, fmaf(g.B, su, quad_c)), 0.f);
+                    acc[col][q] += (u <= grm2) ? gauss : quad;
                   }
-                  acc[col][q] += val;
                 }
               }
             }
@@ -762,7 +772,7 @@ bool paged_serves(const GridArg& g, const float* out) {
   return g.dim % 4 == 0 && g.dim <= kPagedDim && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 }
 
-template <bool BINARY>
+template <bool BINARY, bool CORE>
 hipError_t launch_splat_paged(const GridArg& g, const SortedAtoms& s, int nbatch, float* out,
                               hipStream_t stream) {
   const int dim = g.dim;
@@ -770,13 +780,13 @@ hipError_t launch_splat_paged(const GridArg& g, const SortedAtoms& s, int nbatch
   const int nyp = (dim + 2 * kColXY - 1) / (2 * kColXY);      // waves of a workgroup, <= kPagedWaves
   const long long nitems = (long long)nbatch * nxs * g.ntypes;
   if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, false, 2, true>), dim3((unsigned)nitems),
+  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, false, 2, true, CORE>), dim3((unsigned)nitems),
                      dim3(nyp * kWave), 0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out,
                      nxs, nyp, 1, g.ntypes, 1, kSlabZ, nbatch);
   return hipGetLastError();
 }
 
-template <bool BINARY, bool EXACT, int COLS>
+template <bool BINARY, bool EXACT, int COLS, bool CORE = false>
 hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, float* out,
                         hipStream_t stream) {
   const int dim = g.dim;
@@ -793,7 +803,7 @@ hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, floa
   const long long nitems = (long long)nbatch * nxs * nzs * nyp * nranges;
   if (nitems >= 0x7fffffffll) return hipErrorInvalidValue;
   const int aligned = ((dim % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) ? 1 : 0;
-  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS, false>), dim3((unsigned)nitems), dim3(kWave),
+  hipLaunchKernelGGL((splat_sorted_kernel<BINARY, EXACT, COLS, false, CORE>), dim3((unsigned)nitems), dim3(kWave),
                      0, stream, g, s.slot_info, s.cand, s.records, s.capacity, out, nxs, nyp, nzs,
                      nranges, aligned, slab_z, nbatch);
   return hipGetLastError();
@@ -801,6 +811,8 @@ hipError_t launch_splat(const GridArg& g, const SortedAtoms& s, int nbatch, floa
 
 // 1: grids that the paged write-out serves take it
 std::atomic<int> g_paged{0};
+// 1: Gaussian densities take the kernel instances that skip the exponential for tail-only blocks
+std::atomic<int> g_core_skip{0};
 
 }  // namespace
 
@@ -864,11 +876,14 @@ hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_examp
     if (binary) return launch_splat<true, true, 1>(g, s, nbatch, out, stream);
     return launch_splat<false, true, 1>(g, s, nbatch, out, stream);
   }
+  const bool core = !binary && g_core_skip.load(std::memory_order_relaxed) != 0;
   if (g_paged.load(std::memory_order_relaxed) != 0 && paged_serves(g, out)) {
-    if (binary) return launch_splat_paged<true>(g, s, nbatch, out, stream);
-    return launch_splat_paged<false>(g, s, nbatch, out, stream);
+    if (binary) return launch_splat_paged<true, false>(g, s, nbatch, out, stream);
+    if (core) return launch_splat_paged<false, true>(g, s, nbatch, out, stream);
+    return launch_splat_paged<false, false>(g, s, nbatch, out, stream);
   }
   if (binary) return launch_splat<true, false, 2>(g, s, nbatch, out, stream);
+  if (core) return launch_splat<false, false, 2, true>(g, s, nbatch, out, stream);
   return launch_splat<false, false, 2>(g, s, nbatch, out, stream);
 }
 
@@ -885,5 +900,6 @@ hipError_t launch_forward_sorted(const GridArg& g, const BatchArg& batch, int nb
 }
 
 int set_forward_paged(int on) { return g_paged.exchange(on ? 1 : 0); }
+int set_forward_core_skip(int on) { return g_core_skip.exchange(on ? 1 : 0); }
 
 }  // namespace mg

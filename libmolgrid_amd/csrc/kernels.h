@@ -53,6 +53,7 @@ hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_examp
 // whole 4 KB pages, 0 = one wave per territory writing its own rows.  Same grids bit for bit.
 // Returns the previous setting.
 int set_forward_paged(int on);
+int set_forward_core_skip(int on);
 
 // vector types with per-atom radii, density mode, on the matrix cores (forward_vector_mfma.hip)
 // `workspace` (optional, forward_vector_workspace_bytes()): a launch before the splat leaves the

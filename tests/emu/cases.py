@@ -222,6 +222,7 @@ def group_forward_paged():
     of the per-wave write-out bit for bit: dims 16, 24, 48 and smaller, binary and Gaussian, batches
     with empty examples, output arrays at several alignments inside a 4 KB page."""
     lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    lib.mg_forward_index_core_skip.argtypes = [ctypes.c_int]
     shapes = [(1.0, 15.0, 40, 200), (0.25, 5.75, 2, 15), (0.5, 23.5, 28, 300), (0.5, 3.5, 3, 12),
               (0.5, 1.5, 2, 5), (0.5, 21.5, 5, 150)]
     for res, dimension, ntypes, natoms in shapes:
@@ -238,6 +239,16 @@ def group_forward_paged():
             what = "paged %s binary=%s" % ((res, dimension, ntypes, natoms), binary)
             close(paged, plain, what + " vs per-wave write-out", exact=True)
             close(paged, ref, what + " vs oracle", exact=binary)
+            if not binary:
+                # the instances that skip the exponential in tail-only blocks, with either write-out
+                for paged_on in (0, 1):
+                    lib.mg_forward_index_paged(paged_on)
+                    lib.mg_forward_index_core_skip(1)
+                    skipped = forward_index((res, dimension, binary), center, coords, types, radii, ntypes)
+                    lib.mg_forward_index_paged(0)
+                    lib.mg_forward_index_core_skip(0)
+                    close(skipped, plain, what + ", tail-only blocks without the exponential, paged=%d" % paged_on,
+                          exact=True)
     # a ragged batch with an empty example; the output at offsets of 16, 1040 and 4080 bytes from
     # a page boundary (pages are taken by address)
     cfg = synth.index_batch(2, 4, (30, 120), (3, 9), ntypes=6)

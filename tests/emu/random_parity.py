@@ -135,10 +135,15 @@ def one_round(rng):
     if variant == "cached" or lib.mg_forward_index_workspace_size(ctypes.byref(g0), 1, n, T) <= C.STATIC_BYTES:
         other = C.forward_index(gm_args, center, coords, types, radii, T, variant=variant)
         C.close(other, plain, "forward, %s workspace, " % variant + tag, exact=True)
-    lib.mg_forward_index_paged(1)
-    paged = C.forward_index(gm_args, center, coords, types, radii, T)
-    lib.mg_forward_index_paged(0)
-    C.close(paged, plain, "paged write-out " + tag, exact=True)
+    # the other instances of the splat launch: paged write-out, tail-only blocks without the
+    # exponential, both -- the same grid bit for bit
+    for paged_on, core_on in ((1, 0), (0, 1), (1, 1)):
+        lib.mg_forward_index_paged(paged_on)
+        lib.mg_forward_index_core_skip(core_on)
+        other = C.forward_index(gm_args, center, coords, types, radii, T)
+        lib.mg_forward_index_paged(0)
+        lib.mg_forward_index_core_skip(0)
+        C.close(other, plain, "splat instance paged=%d core_skip=%d, " % (paged_on, core_on) + tag, exact=True)
 
     if True:
         diff = rng.standard_normal(ref.shape).astype(np.float32)
@@ -292,6 +297,7 @@ def main():
     seed = int(sys.argv[2]) if len(sys.argv) > 2 else 1
     first = int(sys.argv[3]) if len(sys.argv) > 3 else 0
     lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    lib.mg_forward_index_core_skip.argtypes = [ctypes.c_int]
     for r in range(first, first + rounds):
         print("round %d of seed %d:" % (r, seed), end=" ")
         one_round(np.random.default_rng([seed, r]))

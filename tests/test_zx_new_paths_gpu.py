@@ -103,6 +103,33 @@ def test_paged_write_out_full_batch(mg, workload, binary):
     assert torch.equal(paged, plain)
 
 
+def test_tail_only_blocks_without_the_exponential_give_the_same_grids(mg, workload):
+    """mg_forward_index_core_skip(1): the kernel instances whose cull marks the blocks that the
+    Gaussian core of an atom can reach and that skip the exponential elsewhere, with either
+    write-out, on ten examples of the benchmark batch: the default instance's grids bit for bit."""
+    from libmolgrid_amd import _capi
+    c = workload
+    B = 10
+    off = c["offsets"][:B + 1]
+    n = int(off[-1])
+    gm = mg.GridMaker(0.5, 23.5)
+    batch = mg.AtomBatch(off)
+    cen, moved, types, radii = dev(c["centers"][:B]), dev(c["moved"][:n]), dev(c["types"][:n]), dev(c["radii"][:n])
+    plain = torch.full((B,) + gm.grid_dimensions(28), 7.0, device="cuda")
+    gm.forward_batch(batch, cen, moved, types, radii, plain)
+    try:
+        for paged in (0, 1):
+            _capi.lib.mg_forward_index_paged(paged)
+            _capi.lib.mg_forward_index_core_skip(1)
+            other = torch.full_like(plain, 6.0)
+            gm.forward_batch(batch, cen, moved, types, radii, other)
+            torch.cuda.synchronize()
+            assert torch.equal(other, plain), "paged=%d" % paged
+    finally:
+        _capi.lib.mg_forward_index_paged(0)
+        _capi.lib.mg_forward_index_core_skip(0)
+
+
 @pytest.mark.parametrize("binary", [False, True])
 def test_atom_lists_give_the_same_grids(mg, binary):
     """mg_forward_vector_ws with its workspace (a launch before the splat lists the atoms that can
