@@ -258,6 +258,39 @@ def one_round(rng):
                                                                (coords[i[0]] - (center - dimension / 2)) / res,
                                                                vr if rti else vr[i[0]], tv[i[0]]))
 
+    # ---- a padded batch of vector-typed examples (every example `width` rows, the rows past its
+    # atoms with zero weights and radius): forward and backward equal the single launches
+    if 2 <= n <= 65 and not rti and d["dim"] <= 33:
+        PB = 3
+        width = n + int(rng.integers(0, 5))
+        counts = [n, int(rng.integers(0, n + 1)), int(rng.integers(1, n + 1))]
+        pc = np.zeros((PB, width, 3), np.float32)
+        pw = np.zeros((PB, width, T), np.float32)
+        pr = np.zeros((PB, width), np.float32)
+        pcen = (center + rng.uniform(-1, 1, (PB, 3))).astype(np.float32)
+        for b, k in enumerate(counts):
+            pc[b, :k], pw[b, :k], pr[b, :k] = coords[:k], tv[:k], vr[:k]
+        pout = E.array((PB, T) + vref.shape[1:], fill=3.0)
+        flat = [E.ptr(E.put(pc.reshape(-1, 3))), E.ptr(E.put(pw.reshape(-1, T))), E.ptr(E.put(pr.reshape(-1)))]
+        assert lib.mg_forward_vector(ctypes.byref(gv), PB, None, width, E.ptr(E.put(pcen)), E.f3((0, 0, 0)),
+                                     flat[0], flat[1], flat[2], T, E.ptr(pout), None) == 0
+        pdiff = rng.standard_normal(pout.shape).astype(np.float32)
+        pag, ptg = E.array((PB * width, 3), fill=9.0), E.array((PB * width, T), fill=9.0)
+        assert lib.mg_backward_vector(ctypes.byref(gv), PB, None, width, E.ptr(E.put(pcen)), E.f3((0, 0, 0)),
+                                      flat[0], flat[1], flat[2], T, E.ptr(E.put(pdiff)), E.ptr(pag),
+                                      E.ptr(ptg), None) == 0
+        for b, k in enumerate(counts):
+            one = np.array(C.forward_vector(vargs, pcen[b], coords[:k], tv[:k], vr[:k])) if k else np.zeros_like(vref)
+            C.close(pout[b], one, "padded vector batch, example %d, " % b + tag, exact=True)
+            if k:
+                a1, t1 = E.array((k, 3), fill=9.0), E.array((k, T), fill=9.0)
+                assert lib.mg_backward_vector(ctypes.byref(gv), 1, None, k, None, E.f3(pcen[b]),
+                                              E.ptr(E.put(coords[:k])), E.ptr(E.put(tv[:k])), E.ptr(E.put(vr[:k])),
+                                              T, E.ptr(E.put(pdiff[b])), E.ptr(a1), E.ptr(t1), None) == 0
+                C.close(pag[b * width:b * width + k], a1, "padded vector backward, atoms, " + tag, exact=True)
+                C.close(ptg[b * width:b * width + k], t1, "padded vector backward, types, " + tag, exact=True)
+            assert not np.asarray(pag[b * width + k:(b + 1) * width]).any(), "gradient of a padding row"
+
     # ---- second order (Gaussian densities only, src/grid_maker.cpp:559), few atoms: the oracle is slow
     if not binary and n <= 65 and d["dim"] <= 33:
         w = rng.standard_normal((n, 3)).astype(np.float32)
