@@ -68,13 +68,15 @@ def one_round(rng):
     common = [nbatch, E.ptr(d_off), width, E.ptr(d_cen), E.f3((0, 0, 0)), E.ptr(d_c)]
     ok = (0, -3)        # MG_OK or MG_ERR_UNSUPPORTED
 
-    for paged in (0, 1):
+    for paged, core in ((0, 0), (1, 0), (0, 1), (1, 1)):      # every instance of the splat launch
         lib.mg_forward_index_paged(paged)
+        lib.mg_forward_index_core_skip(core)
         need = lib.mg_forward_index_workspace_size(ctypes.byref(g), nbatch, width, ntypes)
         ws = E.array(max(need, 1), np.uint8, tight=False)
         assert lib.mg_forward_index_ws(ctypes.byref(g), *common, E.ptr(d_t), E.ptr(d_r), ntypes,
                                        E.ptr(out), E.ptr(ws), need, None) in ok
     lib.mg_forward_index_paged(0)
+    lib.mg_forward_index_core_skip(0)
     for gg, rad in ((g, d_r), (grti, d_tr)):
         need = lib.mg_forward_vector_workspace_size(ctypes.byref(gg), nbatch, width, ntypes)
         ws = E.array(max(need, 1), np.uint8, tight=False)
@@ -123,6 +125,7 @@ if __name__ == "__main__":
     rounds = int(sys.argv[1]) if len(sys.argv) > 1 else 20
     seed = int(sys.argv[2]) if len(sys.argv) > 2 else 0
     lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
+    lib.mg_forward_index_core_skip.argtypes = [ctypes.c_int]
     lib.mg_interpolate_force_gather.argtypes = [ctypes.c_int]
     rng = np.random.default_rng(seed)
     for _ in range(rounds):
