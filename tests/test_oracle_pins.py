@@ -519,6 +519,38 @@ def test_batch_drivers_equal_single_calls():
     assert not out[1].any()
 
 
+def test_index_box_is_half_open_at_the_far_side():
+    """get_bounds_1d (src/grid_maker.cu:66-79) gives [floor((c - r - o) / res), ceil((c + r - o) / res)),
+    and the loops run i < hi: with an atom on a voxel centre and a final radius of exactly five
+    voxels, the voxel five steps DOWN an axis is inside the box (floor of an integer) and the one
+    five steps UP is not (ceil of an integer, exclusive).  For a Gaussian cut off at its radius
+    multiple (no tail) that is visible: exp(-2) on one side, nothing on the other, in the density
+    and, with an upstream gradient of one at both voxels, as a net pull in the gradient."""
+    res, dim = 0.5, 24
+    g = oracle.GridMaker(res, (dim - 1) * res, gaussian_radius_multiple=-1.0)
+    assert g.p.final_radius_multiple == 1.0 and g.p.gaussian_radius_multiple == 1.0
+    m = dim // 2
+    half = (dim - 1) * res / 2
+    atom = np.array([[m * res - half] * 3], np.float32)
+    types, radii = np.zeros(1, np.float32), np.full(1, 2.5, np.float32)
+    lo, hi = g.bounds_1d(-half, float(atom[0, 0]), 2.5)
+    assert (lo, hi) == (m - 5, m + 5)                       # half open: m + 5 itself is outside
+    d = g.forward((0, 0, 0), atom, types, radii, 1)[0]
+    assert d[m, m, m] == 1.0
+    for axis in range(3):
+        down, up = [m, m, m], [m, m, m]
+        down[axis] -= 5
+        up[axis] += 5
+        assert d[tuple(down)] == pytest.approx(E2, rel=1e-6) and d[tuple(up)] == 0.0
+    # every other voxel at distance 2.5 -- (3, 4, 0) steps and permutations -- lies inside the box
+    assert d[m + 3, m + 4, m] == pytest.approx(E2, rel=1e-6) and d[m + 4, m, m + 3] == pytest.approx(E2, rel=1e-6)
+    diff = np.zeros((1, dim, dim, dim), np.float32)
+    diff[0, m - 5, m, m] = diff[0, m + 5, m, m] = 1.0
+    grad = g.backward((0, 0, 0), atom, types, radii, diff)[0]
+    # only the voxel at -5 counts: -(dx / dist) * (-4 dist / ar^2 exp(-2)) with dx = -2.5, dist = ar = 2.5
+    assert grad[0] == pytest.approx(-4.0 / 2.5 * E2, rel=1e-6) and grad[1] == 0 and grad[2] == 0
+
+
 def test_oracle_is_clean_under_address_and_ub_sanitizers():
     """`make -C oracle asan`: every entry point of the oracle over the edge cases of its loops
     (atoms outside the grid and on its faces, radii <= 0, ignored types, no atoms, a one-voxel
