@@ -150,6 +150,9 @@ def test_python_host_layer_on_a_fake_device(emulated_library):
     kernels behind the C ABI) against the oracle: forward overloads, workspaces, the sort and splat
     halves, backward with the fused un-rotation, vector types with atom lists, autograd, resampling."""
     assert "comparisons passed" in _run("python_layer.py")
+    # and with the grid maker, the molecule and the way of calling drawn at random (host arrays,
+    # float64 grids, ragged batches whose workspaces must grow, radii by type, the autograd layer)
+    assert "comparisons passed" in _run("random_python_layer.py", "10", "3")
 
 
 def test_smoke_and_bench_run_end_to_end_on_a_fake_device(emulated_library):
