@@ -4,7 +4,8 @@ binary, radius scale, radius multiple), a molecule, and the way the call is made
 host arrays or float64 grids; a single example, a padded batch or a ragged batch whose AtomBatch is
 reused with a larger batch afterwards (its cached workspaces must grow); index or vector types,
 radii by atom or by type; backward with and without the fused un-rotation; the autograd layer with
-one example and with a padded batch.  ``python tests/emu/random_python_layer.py [rounds] [seed]``."""
+one example and with a padded batch; the overloads of GridInterpolater; Transform on device and
+host arrays.  ``python tests/emu/random_python_layer.py [rounds] [seed]``."""
 import os
 import sys
 
@@ -124,6 +125,43 @@ def one_round(rng):
         close(xb.grad[0], ra, "batched Coords2Grid backward " + tag, rtol=1e-4, atol=5e-5)
         close(xb.grad[1], 0.5 * xb.grad[0].numpy(), "batched Coords2Grid backward, half weights, " + tag,
               rtol=1e-5, atol=1e-5)
+
+    # ---- resampling: the three overloads of one grid, and a batch; Transform on device and on host --
+    if dim <= 16 and T <= 8:
+        q = synth.random_quaternions(rng, 1)[0]
+        rc = rng.uniform(-1, 1, 3).astype(np.float32)
+        tr = rng.uniform(-1.5, 1.5, 3).astype(np.float32)
+        t = mg.Transform(mg.Quaternion(*q), tuple(rc), tuple(tr))
+        out_res = float(rng.choice([res, res * 0.5, res * 1.5]))
+        out_dim = int(rng.choice([dim, dim + 3, max(dim - 2, 1)]))
+        gi = mg.GridInterpolater(res, dimension, out_res, (out_dim - 1) * out_res)
+        src = ref if not binary else rng.standard_normal(ref.shape).astype(np.float32)
+        dst = torch.full((T, out_dim, out_dim, out_dim), 9.0, device="cuda")
+        gi.forward(as_input(rng, src), t, dst)
+        one = oracle.interpolate_batch(res, dimension, out_res, (out_dim - 1) * out_res, rc[None], src[None],
+                                       q[None], rc[None], tr[None], rc[None])[0]
+        close(dst, one, "GridInterpolater.forward(in, transform, out) " + tag)
+        ic, oc = rng.uniform(-1, 1, 3).astype(np.float32), rng.uniform(-1, 1, 3).astype(np.float32)
+        gi.forward(tuple(ic), dev(src), t, tuple(oc), dst)
+        close(dst, oracle.interpolate_batch(res, dimension, out_res, (out_dim - 1) * out_res, ic[None], src[None],
+                                            q[None], rc[None], tr[None], oc[None])[0],
+              "GridInterpolater.forward with centres " + tag)
+        B = 3
+        qs = synth.random_quaternions(rng, B)
+        cs, ts = rng.uniform(-1, 1, (B, 3)).astype(np.float32), rng.uniform(-2, 2, (B, 3)).astype(np.float32)
+        srcs = np.stack([src, src[:, ::-1].copy(), 2 * src]).astype(np.float32)
+        dsts = torch.full((B, T, out_dim, out_dim, out_dim), 9.0, device="cuda")
+        gi.forward_batch(dev(srcs), as_input(rng, qs), as_input(rng, cs), as_input(rng, ts), dsts)
+        close(dsts, oracle.interpolate_batch(res, dimension, out_res, (out_dim - 1) * out_res, cs, srcs, qs, cs, ts, cs),
+              "GridInterpolater.forward_batch " + tag)
+        a, b = torch.empty((n, 3), device="cuda"), np.empty((n, 3), np.float32)
+        t.forward(dev(coords), a)
+        t.forward(coords, b)
+        close(a, b, "Transform.forward on the device and on the host " + tag, exact=True)
+        close(b, oracle.transform_forward(q, rc, tr, coords), "Transform.forward against the oracle " + tag, exact=True)
+        t.backward(dev(b), a)
+        t.backward(b.copy(), b)
+        close(a, b, "Transform.backward on the device and on the host " + tag, exact=True)
 
 
 def main():
