@@ -13,13 +13,14 @@ def pytest_configure(config):
 
 
 # GPU tests whose kernels are re-written sweeps and scans (vector-typed forward with atom lists,
-# vector backward, relevance, second order, and the layers on top of them) run after the tests of
+# vector backward, relevance, second order, and the layers on top of them), and tests of behaviour
+# that is newer than the last GPU run (radii <= 0 dropped in the sort), run after the tests of
 # the paths whose machine code is the one that has already passed on a GPU, or close to it: under
 # `pytest -x` a failure among the former then cannot hide the results of the latter.  The two files
 # whose names sort last keep their places at the end.
 LATER = ("test_vector_gpu.py", "test_second_order_gpu.py", "test_torch_gpu.py", "test_cpp_api.py",
          "test_vector_types_full_size", "test_forward_vector_and_batches_into_double_grids",
-         "test_vector_typed_examples", "test_training_")
+         "test_vector_typed_examples", "test_training_", "test_zero_and_negative_radii")
 
 
 def _tier(item):
