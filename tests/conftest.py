@@ -20,7 +20,8 @@ def pytest_configure(config):
 # whose names sort last keep their places at the end.
 LATER = ("test_vector_gpu.py", "test_second_order_gpu.py", "test_torch_gpu.py", "test_cpp_api.py",
          "test_vector_types_full_size", "test_forward_vector_and_batches_into_double_grids",
-         "test_vector_typed_examples", "test_training_", "test_zero_and_negative_radii")
+         "test_vector_typed_examples", "test_training_", "test_zero_and_negative_radii",
+         "test_backward_gpu.py::test_unusual_radius_multiples[gm_args0]")   # the kernel instance for a Gaussian without a tail
 
 
 def _tier(item):
