@@ -297,6 +297,9 @@ class Workload(object):
         self.diff = torch.randn((B, T, D, D, D), device="cuda", generator=gen)
         self.grads = torch.empty_like(self.coords)
         self.side = None
+        # True: the backward launch also takes the gradients back through the example's rotation
+        # (mg_backward_index_unrotated: one launch instead of two, the same floats bit for bit)
+        self.fused_unrotation = False
 
     def k_transform(self):
         self.mg.transform_batch(self.offsets, self.quats, self.centers, self.trans, self.coords,
@@ -327,8 +330,14 @@ class Workload(object):
         # launch, bit for bit; it measures the same, see kernels.backward.unrotated_ms)
         self.k_transform()
         self.k_forward()
-        self.k_backward()
-        self.k_unrotate()
+        self.backward_and_unrotation()
+
+    def backward_and_unrotation(self):
+        if self.fused_unrotation:
+            self.k_backward_unrotated()
+        else:
+            self.k_backward()
+            self.k_unrotate()
 
     def step_overlapped(self):
         # The forward and the backward pass of a step do not depend on each other, and the
@@ -347,10 +356,14 @@ class Workload(object):
             sb = self.gm.sort_batch(self.offsets, self.centers, self.moved, self.types, self.radii,
                                     self.T)
             self.ev_sorted.record(self.side)
-        self.k_backward()
+        if self.fused_unrotation:
+            self.k_backward_unrotated()
+        else:
+            self.k_backward()
         main.wait_event(self.ev_sorted)
         self.gm.splat_batch(sb, self.grid)
-        self.k_unrotate()
+        if not self.fused_unrotation:
+            self.k_unrotate()
 
     def timed(self, run):
         """(ms per step, ms per step the host needs to enqueue) over exactly --steps steps after
@@ -449,6 +462,7 @@ def run_candidates(args):
     # 2. the other instances of the splat launch -- the paged write-out, tail-only blocks without
     # the exponential, both --: their grids bit for bit, the forward call's time with each, and
     # the store skeleton of either write-out (the same call with every atom ignored)
+    valid, check, fastest = [], {}, None
     if not args.no_autotune:
         check = {"identical": {}}
         try:
@@ -484,6 +498,15 @@ def run_candidates(args):
                 select(fastest)
                 step_variants(fastest + "/", True)
                 select("per_wave")
+    # 4. the un-rotation of the gradients inside the backward launch (four launches a step instead
+    # of five), with the default instance and with the fastest one
+    w.fused_unrotation = True
+    step_variants("fused_unrotation/", True)
+    if not args.no_autotune and valid and "per_wave_ms" in check and check[fastest + "_ms"] < check["per_wave_ms"]:
+        select(fastest)
+        step_variants(fastest + "+fused_unrotation/", True)
+        select("per_wave")
+    w.fused_unrotation = False
     emit({"done": True})
 
 
@@ -734,7 +757,9 @@ def main():
     if child_note is not None:
         step_variants["candidates_note"] = child_note
     if write_out is not None:
-        used = best.split("/")[0] if "/" in best else "per_wave"
+        used = best.split("/")[0].split("+")[0] if "/" in best else "per_wave"
+        if used == "fused_unrotation":
+            used = "per_wave"
         write_out["used"] = used
         if used != "per_wave" and dominant_fwd and (used + "_ms") in write_out:
             # `value` is from a step whose splat launch is another instance of the kernel (same grids
@@ -759,7 +784,8 @@ def main():
         # which way of enqueueing the step `value` is from (step_variants lists all of them):
         # serial = the reference's order on one stream, overlapped = the sort launch beside the
         # backward pass; eager = launch by launch, graph = one captured HIP graph; a prefix such as
-        # "paged/" = with that instance of the splat launch (forward_write_out lists them)
+        # "paged/" = with that instance of the splat launch (forward_write_out lists them),
+        # "fused_unrotation" = the gradients' un-rotation inside the backward launch
         "launch": best,
         "ms_per_step": round(ms_per_step, 4),
         # wall time the host needs to enqueue a step (the timed loop before its synchronize): when
