@@ -203,9 +203,21 @@ def other_workloads(mg, synth, gm, offsets, centers, moved, types, radii, grid, 
         out = torch.empty((VB,) + gv.grid_dimensions(28), device="cuda")
         ms = event_ms(lambda: gv.forward_batch(ab, vcen, vc, vt, vr, out), 5)
         nbytes = out.numel() * 4 + vc.shape[0] * (16 + 4 * 28)
-        res["forward_vector_binary" if binary else "forward_vector"] = entry(
-            ms, nbytes, grids_per_s=round(VB / (ms * 1e-3), 1),
-            workload="configs[3]: %d x %d atoms, 28x96^3 at 0.25 A" % (VB, VN))
+        key = "forward_vector_binary" if binary else "forward_vector"
+        res[key] = entry(ms, nbytes, grids_per_s=round(VB / (ms * 1e-3), 1),
+                         workload="configs[3]: %d x %d atoms, 28x96^3 at 0.25 A" % (VB, VN))
+        try:
+            # the same call without the per-slab atom lists (every workgroup scans every atom of its
+            # example): the plain entry point of the C ABI, which takes no workspace
+            from libmolgrid_amd import _capi
+            off32 = ab.dev
+            call = lambda: _capi.check(_capi.lib.mg_forward_vector(
+                gv._p, VB, off32.data_ptr(), ab.largest, vcen.data_ptr(), _capi.f3((0, 0, 0)),
+                vc.data_ptr(), vt.data_ptr(), vr.data_ptr(), 28, out.data_ptr(),
+                torch.cuda.current_stream().cuda_stream), "mg_forward_vector")
+            res[key]["without_atom_lists_ms"] = round(event_ms(call, 5), 4)
+        except Exception as e:      # a new measurement must not cost the bench line
+            res[key]["without_atom_lists_ms"] = repr(e)[:200]
         del out
     try:
         # backward pass for vector types on the same atoms (atom and type gradients): the upstream
