@@ -27,13 +27,26 @@ f3, f4 = _capi.f3, _capi.f4
 _keep = []
 
 
+# Number of 4-byte elements by which arrays of 4-byte elements start past a 16-byte boundary (0..3):
+# callers hand the library views into larger tensors, whose first element sits anywhere.
+MISALIGN = 0
+
+
 def array(shape, dtype=np.float32, fill=None, tight=True):
     """Uninitialised (0xCB bytes) array in guarded memory."""
     shape = tuple(int(d) for d in np.atleast_1d(shape))
-    n = int(np.prod(shape)) * np.dtype(dtype).itemsize
-    p = (lib.emu_alloc_tight if tight else lib.emu_alloc)(max(n, 1))
-    buf = (ctypes.c_char * max(n, 1)).from_address(p)
-    a = np.frombuffer(buf, dtype=dtype, count=int(np.prod(shape))).reshape(shape)
+    item = np.dtype(dtype).itemsize
+    n = int(np.prod(shape)) * item
+    # (a tight block ends within 15 bytes of the guard page: shifting the array's start by
+    # 4 * MISALIGN bytes keeps that, as the size is rounded up to 16 bytes first)
+    shift = 4 * MISALIGN if (tight and item == 4) else 0
+    total = max(n, 1) + (16 if shift else 0)
+    if shift:
+        total = (total + 15) & ~15
+    p = (lib.emu_alloc_tight if tight else lib.emu_alloc)(total)
+    buf = (ctypes.c_char * total).from_address(p)
+    start = ((total - n - shift) // 16) * 16 + shift if shift else 0      # as far back as it goes
+    a = np.frombuffer(buf, dtype=dtype, count=int(np.prod(shape)), offset=start).reshape(shape)
     _keep.append(buf)
     if fill is not None:
         a[...] = fill

@@ -333,6 +333,8 @@ def main():
     lib.mg_forward_index_core_skip.argtypes = [ctypes.c_int]
     for r in range(first, first + rounds):
         print("round %d of seed %d:" % (r, seed), end=" ")
+        # (the arrays of this round start 0 to 12 bytes past a 16-byte boundary)
+        E.MISALIGN = int(np.random.default_rng([seed, r, 1]).choice([0, 0, 1, 2, 3]))
         one_round(np.random.default_rng([seed, r]))
         E.release_all()
     print("random parity: %d rounds passed" % rounds)
