@@ -53,7 +53,7 @@ def test_one_unit_in_the_last_place_of_the_approximate_instructions(emulated_lib
     notice at all, sums stay within twice the tolerance (tests/emu/cases.py)."""
     env = dict(os.environ, EMU_APPROX="hash")
     for args in (["cases.py", "forward_index"], ["cases.py", "backward_index"], ["cases.py", "interpolate"],
-                 ["random_parity.py", "15", "9"], ["random_resample.py", "10", "9"]):
+                 ["random_parity.py", "10", "9"], ["random_resample.py", "8", "9"]):
         p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
@@ -67,7 +67,7 @@ def test_threads_and_workgroups_run_last_to_first(emulated_library):
     workgroup starts, so neither zeros nor the previous workgroup's leftovers can be relied on.)"""
     env = dict(os.environ, EMU_ORDER="reverse")
     for args in (["cases.py", "forward_batch"], ["cases.py", "forward_vector"], ["cases.py", "second_order"],
-                 ["cases.py", "interpolate"], ["random_parity.py", "12", "6"]):
+                 ["cases.py", "interpolate"], ["random_parity.py", "8", "6"]):
         p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
@@ -81,7 +81,7 @@ def test_with_fused_multiply_adds(emulated_library):
     wherever it matters."""
     env = dict(os.environ, EMU_CONTRACT="1")
     for args in (["cases.py", "transform"], ["cases.py", "forward_index"], ["cases.py", "backward_index"],
-                 ["random_parity.py", "15", "8"]):
+                 ["random_parity.py", "10", "8"]):
         p = subprocess.run([sys.executable, os.path.join(HERE, "emu", args[0])] + args[1:], env=env,
                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
         assert p.returncode == 0 and "passed" in p.stdout, "%s:\n%s" % (" ".join(args), p.stdout[-3000:])
@@ -105,14 +105,14 @@ def test_randomised_parity(emulated_library):
     with radii that put voxels ON the cut-off -- and every kernel compared with the oracle under
     the GPU tests' bounds (a few rounds here; thousands by hand, which is how the handling of a
     Gaussian cut off without a tail and of a binary sphere as wide as its index box was found)."""
-    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_parity.py"), "30", "5"],
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_parity.py"), "20", "5"],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
-    assert p.returncode == 0 and "30 rounds passed" in p.stdout, p.stdout[-3000:]
+    assert p.returncode == 0 and "20 rounds passed" in p.stdout, p.stdout[-3000:]
     # the same for resampling: grid sizes, resolution ratios, centres, shifts beyond the input,
     # axis-aligned and random rotations (tests/emu/random_resample.py; 1,800 rounds by hand)
-    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_resample.py"), "30", "5"],
+    p = subprocess.run([sys.executable, os.path.join(HERE, "emu", "random_resample.py"), "20", "5"],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=1500)
-    assert p.returncode == 0 and "30 rounds passed" in p.stdout, p.stdout[-3000:]
+    assert p.returncode == 0 and "20 rounds passed" in p.stdout, p.stdout[-3000:]
 
 
 @pytest.mark.parametrize("checks", ["undefined", "address"])
@@ -127,7 +127,7 @@ def test_run_time_checks(emulated_library, checks):
     env = dict(os.environ, EMU_SANITIZE="1" if checks == "undefined" else "address",
                ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0")
     groups = [["cases.py", "forward_paged"], ["cases.py", "backward_index"], ["cases.py", "second_order"],
-              ["cases.py", "interpolate"], ["random_parity.py", "10", "4"], ["fuzz.py", "6", "5"]]
+              ["cases.py", "interpolate"], ["random_parity.py", "6", "4"], ["fuzz.py", "6", "5"]]
     if checks == "undefined":
         groups.insert(2, ["cases.py", "forward_vector"])
     for args in groups:
@@ -152,7 +152,7 @@ def test_python_host_layer_on_a_fake_device(emulated_library):
     assert "comparisons passed" in _run("python_layer.py")
     # and with the grid maker, the molecule and the way of calling drawn at random (host arrays,
     # float64 grids, ragged batches whose workspaces must grow, radii by type, the autograd layer)
-    assert "comparisons passed" in _run("random_python_layer.py", "10", "3")
+    assert "comparisons passed" in _run("random_python_layer.py", "6", "3")
 
 
 def test_smoke_and_bench_run_end_to_end_on_a_fake_device(emulated_library):
