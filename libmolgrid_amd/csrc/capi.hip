@@ -152,7 +152,11 @@ int mg_gridmaker_init(mg_gridmaker* g, float resolution, float dimension, int bi
     g->gaussian_radius_multiple = grm;
     g->final_radius_multiple = (1 + 2 * grm * grm) / (2 * grm);
   }
-  g->dim = (uint32_t)(std::round(dimension / resolution) + 1);
+  // (the reference's arithmetic, include/libmolgrid/grid_maker.h; a quotient that is not a number
+  // or out of range must not reach the conversion: such a grid maker gets dim = 0, which every
+  // entry point rejects)
+  const float points = std::round(dimension / resolution) + 1;
+  g->dim = (points >= 1.f && points <= 65535.f) ? (uint32_t)points : 0u;
   // Quadratic a*(d/r)^2 + b*(d/r) + c matching value and slope of the Gaussian
   // at d = grm*r and reaching zero with zero slope at the final multiple; the
   // exponential is taken in double and the results are stored as float.
@@ -602,11 +606,14 @@ int mg_interpolate(float in_resolution, float in_dimension, float out_resolution
   p.in_half = (float)(in_dimension / 2.0);
   p.out_half = (float)(out_dimension / 2.0);
   // include/libmolgrid/grid_interpolater.h:59-64
-  p.in_dim = (int)(std::round(in_dimension / in_resolution) + 1);
-  p.out_dim = (int)(std::round(out_dimension / out_resolution) + 1);
-  p.channels = channels;
-  if (p.in_dim <= 0 || p.out_dim <= 0 || p.in_dim > 1200 || p.out_dim > 1200)
+  const float in_points = std::round(in_dimension / in_resolution) + 1;
+  const float out_points = std::round(out_dimension / out_resolution) + 1;
+  // (also false for a quotient that is not a number, which must not reach the conversion)
+  if (!(in_points >= 1.f && in_points <= 1200.f && out_points >= 1.f && out_points <= 1200.f))
     return MG_ERR_OUT_OF_RANGE;
+  p.in_dim = (int)in_points;
+  p.out_dim = (int)out_points;
+  p.channels = channels;
   return from_hip(launch_interpolate(p, nbatch, vec3(in_centers, in_center_host), in,
                                      vec4(quats, quat_host), vec3(rot_centers, rot_center_host),
                                      vec3(translations, translation_host),

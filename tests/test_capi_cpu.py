@@ -46,6 +46,21 @@ def test_error_strings(mg):
         _capi.check(1, "x")
 
 
+@pytest.mark.parametrize("resolution,dimension", [
+    (0.0, 5.0), (float("nan"), 5.0), (0.5, float("nan")), (0.5, float("inf")), (1e-30, 1e30), (-1.0, 5.0)])
+def test_grid_sizes_that_are_not_numbers_give_a_grid_maker_nothing_accepts(resolution, dimension):
+    """dimension / resolution that is not a number, infinite or beyond any grid must not reach the
+    conversion to an integer: the grid maker gets dim = 0, which every entry point rejects."""
+    import ctypes
+    from libmolgrid_amd import _capi
+    g = _capi.mg_gridmaker()
+    assert _capi.lib.mg_gridmaker_init(ctypes.byref(g), resolution, dimension, 0, 0, 1.0, 1.0) == 0
+    assert g.dim == 0
+    code = _capi.lib.mg_forward_index(ctypes.byref(g), 1, None, 0, None, _capi.f3((0, 0, 0)), None, None,
+                                      None, 1, None, None)
+    assert code < 0
+
+
 @pytest.mark.parametrize("args", [
     (0.5, 23.5, False, False, 1.0, 1.0), (0.25, 23.75, True, False, 1.0, 1.0),
     (0.1, 6.0, False, True, 0.5, 3.0), (0.5, 11.5, False, False, 1.3, -1.5),
