@@ -337,6 +337,8 @@ int mg_forward_index(const mg_gridmaker* g, int nbatch, const int32_t* atom_offs
                                     radii, ntypes, out, &nothing);
   if (s != MG_OK || nothing) return s;
   const size_t need = mg_forward_index_workspace_size(g, nbatch, atoms_per_example, ntypes);
+  // (before anything is allocated: sizes that the launches do not cover)
+  if (!forward_sorted_supports(grid_arg(g, ntypes), nbatch, atoms_per_example)) return MG_ERR_UNSUPPORTED;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return from_hip(e);

@@ -823,21 +823,28 @@ size_t forward_sorted_workspace_bytes(int nbatch, int atoms_per_example, int nty
          (size_t)capacity * 16;
 }
 
+// The sizes the two launches address with 32 bits: a channel below 4 GB, the records of the batch
+// below 4 GB, the table of (channel, x slab) keys below 2^26 entries.
+bool forward_sorted_supports(const GridArg& g, int nbatch, int per_example) {
+  const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
+  if (chan_stride * 4 >= 0xfffffff0ull) return false;
+  if ((long long)nbatch * per_example * 16 >= 0xfffffff0ll) return false;
+  const int nxs = (g.dim + kColXY - 1) / kColXY;
+  return (long long)g.ntypes * nxs < (1 << 26);
+}
+
 namespace {
 
 // hipErrorInvalidValue = the case is not covered (a channel of 4 GB or more, more records than a
 // buffer addresses, a workspace that is too small).
 hipError_t sorted_layout(const GridArg& g, int nbatch, int per_example, void* workspace,
                          size_t workspace_bytes, SortedAtoms* s, int* nxs_out) {
-  const size_t chan_stride = (size_t)g.dim * g.dim * g.dim;
-  if (chan_stride * 4 >= 0xfffffff0ull) return hipErrorInvalidValue;
+  if (!forward_sorted_supports(g, nbatch, per_example)) return hipErrorInvalidValue;
   const long long capacity = (long long)nbatch * per_example;
-  if (capacity * 16 >= 0xfffffff0ll) return hipErrorInvalidValue;
   if (workspace == nullptr ||
       workspace_bytes < forward_sorted_workspace_bytes(nbatch, per_example, g.ntypes, g.dim))
     return hipErrorInvalidValue;
   const int nxs = (g.dim + kColXY - 1) / kColXY;
-  if ((long long)g.ntypes * nxs >= (1 << 26)) return hipErrorInvalidValue;
   *s = carve(workspace, nbatch, g.ntypes * nxs, capacity);
   *nxs_out = nxs;
   return hipSuccess;

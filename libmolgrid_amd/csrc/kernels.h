@@ -52,6 +52,7 @@ hipError_t launch_splat_sorted(const GridArg& g, int nbatch, int atoms_per_examp
 // float4 pieces: 1 = workgroups that own a slab of four x planes of one channel and write it as
 // whole 4 KB pages, 0 = one wave per territory writing its own rows.  Same grids bit for bit.
 // Returns the previous setting.
+bool forward_sorted_supports(const GridArg& g, int nbatch, int per_example);
 int set_forward_paged(int on);
 int set_forward_core_skip(int on);
 
