@@ -121,12 +121,36 @@ def one_round(rng):
     lib.mg_interpolate_force_gather(0)
 
 
+def extreme_scalars():
+    """Batch sizes, atom counts and channel counts of zero, one, minus one and 2^31 - 1 with no arrays
+    at all: the size functions must not overflow and every launching entry point must refuse."""
+    big = 2 ** 31 - 1
+    z3, q1 = E.f3((0, 0, 0)), E.f4((1, 0, 0, 0))
+    for res, dimension in ((0.5, 3.5), (0.001, 65.0), (0.5, 32767.0)):
+        g = E.gridmaker(res, dimension)
+        for nb in (0, 1, big):
+            for per in (0, 1, big):
+                for ntypes in (0, 1, big):
+                    lib.mg_forward_index_workspace_size(ctypes.byref(g), nb, per, ntypes)
+                    lib.mg_forward_vector_workspace_size(ctypes.byref(g), nb, per, ntypes)
+        for nb, per, ntypes in ((big, big, big), (-1, 1, 1), (1, -1, 1), (1, 1, -1), (big, 1, 1)):
+            codes = [
+                lib.mg_forward_index(ctypes.byref(g), nb, None, per, None, z3, None, None, None, ntypes, None, None),
+                lib.mg_backward_index(ctypes.byref(g), nb, None, per, None, z3, None, None, None, ntypes, None,
+                                      None, None),
+                lib.mg_forward_vector(ctypes.byref(g), nb, None, per, None, z3, None, None, None, ntypes, None, None),
+                lib.mg_transform_forward(nb, None, per, None, q1, None, z3, None, z3, 1, None, None, None)]
+            assert all(c < 0 for c in codes), (nb, per, ntypes, codes)
+    print("fuzz: extreme scalar arguments refused", flush=True)
+
+
 if __name__ == "__main__":
     rounds = int(sys.argv[1]) if len(sys.argv) > 1 else 20
     seed = int(sys.argv[2]) if len(sys.argv) > 2 else 0
     lib.mg_forward_index_paged.argtypes = [ctypes.c_int]
     lib.mg_forward_index_core_skip.argtypes = [ctypes.c_int]
     lib.mg_interpolate_force_gather.argtypes = [ctypes.c_int]
+    extreme_scalars()
     rng = np.random.default_rng(seed)
     for _ in range(rounds):
         one_round(rng)
